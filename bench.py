@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused logprob + GRPO loss head path (forward + backward).
+
+One step = one packed micro-batch through: fused lm_head forward (logprob,
+entropy, lse), the policy-loss kernel (loss sums + per-token upstream grads) and
+the fused backward (dhidden bf16, dW fp32).  Default workload: the Qwen3-8B head
+(H=4096, V=151936, bf16) on a 16384-token micro-batch, inputs resident in HBM.
+
+Prints ONE JSON line:  metric/value/unit per the driver contract, plus
+  roofline     - the forward kernel against the bf16 MFMA peak (HIP-event timed, live)
+  cpu_baseline - the torch oracle (reference op order) timed on the host cores on a row sample
+and some extra, clearly named fields (per-stage times, the unfused torch-on-GPU path).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from chatlearn_amd import ops, synthetic  # noqa: E402
+from chatlearn_amd._lib import LOSS_GRPO, LOSS_GSPO  # noqa: E402
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3
+
+
+def build_workload(cfg, device):
+    gen = synthetic.generator_for(cfg)
+    samples = synthetic.fill_microbatch(cfg, synthetic.sample_population(cfg, gen))
+    cu, mask = synthetic.packed_layout(samples)
+    T = int(cu[-1])
+    hidden, weight, labels = synthetic.make_head_tensors(cfg, T, gen, device=device, device_generate=True)
+    return samples, cu.to(device), mask.to(device), T, hidden, weight, labels
+
+
+def advantages_for(samples, device):
+    """Group mean/std advantages through the library's AdvantageComputer mirror."""
+    from chatlearn_amd.algorithm.grpo_utils.advantage_compute import AdvantageComputer
+
+    class _Buf:
+        def __init__(self, b):
+            self.buffer = b
+    pop = [dict(s) for s in samples]
+    AdvantageComputer(num_inference_per_prompt=1 << 30)([_Buf(pop)])
+    return torch.tensor([float(s["advantages"]) for s in pop], dtype=torch.float32, device=device)
+
+
+def cpu_baseline(cfg, rows, threads):
+    """The oracle (torch, reference op order: linear -> log_softmax+gather -> chunked entropy ->
+    GRPO/GSPO loss -> masked sums -> backward) on the host cores, fp32, on `rows` packed tokens."""
+    from oracle import losses as ol
+    from oracle import softmax_stats as osm
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(cfg.seed)
+    hidden = torch.randn(rows, cfg.H, generator=g).requires_grad_(cfg.loss is not None)
+    weight = (torch.randn(cfg.V, cfg.H, generator=g) * cfg.w_std).requires_grad_(cfg.loss is not None)
+    labels = torch.randint(0, cfg.V, (1, rows), generator=g)
+    old = torch.full((1, rows), -12.0)
+    ref = torch.full((1, rows), -12.0)
+    mask = torch.ones(1, rows, dtype=torch.int32)
+
+    def step():
+        logits = torch.nn.functional.linear(hidden, weight).unsqueeze(0) / cfg.temperature
+        lp = osm.logprobs_from_logits(logits, labels)
+        if cfg.loss is None:
+            with torch.no_grad():
+                osm.entropy_from_logits_with_chunking(logits)
+            return
+        ctx = torch.enable_grad() if cfg.entropy_coef > 0 else torch.no_grad()
+        with ctx:
+            ent = osm.entropy_from_logits_with_chunking(logits)
+        total, _ = ol.fsdp_policy_loss(lp, ent, old, ref, [0.5], mask, float(rows), entropy_coef=cfg.entropy_coef,
+                                       kl_coef=cfg.kl_coef, pos_clip_ratio=cfg.pos_clip_ratio,
+                                       neg_clip_ratio=cfg.neg_clip_ratio, final_clip_ratio=cfg.final_clip_ratio,
+                                       use_group_sequence_policy=(cfg.loss == "gspo"))
+        total.backward()
+        hidden.grad = None
+        weight.grad = None
+
+    ctx = torch.no_grad() if cfg.loss is None else torch.enable_grad()
+    with ctx:
+        step()  # warm-up
+        t0 = time.perf_counter()
+        reps = 0
+        while reps < 2 or time.perf_counter() - t0 < 10.0:
+            step()
+            reps += 1
+            if time.perf_counter() - t0 > 30.0:
+                break
+        dt = (time.perf_counter() - t0) / reps
+    return rows / dt, reps
+
+
+def unfused_gpu(cfg, hidden, weight, labels, old, ref, adv, cu, mask, n_tok, steps):
+    """What the reference's FSDP trainer does today, on the same GPU in bf16: materialised logits,
+    log_softmax + gather, chunked entropy, re-padding to [B,S], torch loss ops, autograd backward
+    (policy_trainer.py:216-286)."""
+    from oracle import indexing as oi
+    from oracle import losses as ol
+    from oracle import softmax_stats as osm
+    h = hidden.detach().clone().requires_grad_(True)
+    w = weight.detach().clone().requires_grad_(True)
+    lab = labels.view(1, -1)
+    lens = (cu[1:] - cu[:-1]).long()
+    B, S = lens.numel(), int(lens.max())
+    ar = torch.arange(S, device=hidden.device)
+    attn = (ar.unsqueeze(0) < lens.unsqueeze(1))
+    indices = torch.nonzero(attn.flatten(), as_tuple=False).flatten()
+    pad = lambda x: oi.pad_input(x.unsqueeze(-1), indices, B, S).squeeze(-1)
+    old_p, ref_p, mask_p = pad(old), pad(ref), pad(mask)
+    adv_list = adv.tolist()
+
+    def step():
+        logits = torch.nn.functional.linear(h, w).unsqueeze(0)
+        if cfg.temperature != 1.0:
+            logits = logits / cfg.temperature
+        lp = osm.logprobs_from_logits(logits, lab)
+        with (torch.enable_grad() if cfg.entropy_coef > 0 else torch.no_grad()):
+            ent = osm.entropy_from_logits_with_chunking(logits)
+        total, _ = ol.fsdp_policy_loss(pad(lp[0].float()), pad(ent[0]), old_p, ref_p, adv_list, mask_p, n_tok,
+                                       entropy_coef=cfg.entropy_coef, kl_coef=cfg.kl_coef,
+                                       pos_clip_ratio=cfg.pos_clip_ratio, neg_clip_ratio=cfg.neg_clip_ratio,
+                                       diff_clip_ratio=cfg.diff_clip_ratio, final_clip_ratio=cfg.final_clip_ratio,
+                                       use_group_sequence_policy=(cfg.loss == "gspo"))
+        total.backward()
+        h.grad = None
+        w.grad = None
+
+    step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c2", choices=sorted(synthetic.CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-unfused", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=256)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives are built); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    cfg = synthetic.CONFIGS[args.config]
+    samples, cu, mask, T, hidden, weight, labels = build_workload(cfg, dev)
+    train = cfg.loss is not None
+    n_tok = float(mask.sum().item())
+    adv = advantages_for(samples, dev)
+
+    # old / ref logprobs around the model's own logprob, as the recipe says
+    lp0, *_ = ops.lmhead_forward(hidden, weight, labels, cfg.temperature, need_entropy=False)
+    old, ref = synthetic.noisy_logprobs(lp0, synthetic.generator_for(cfg))
+    dweight = torch.zeros(cfg.V, cfg.H, dtype=torch.float32, device=dev) if train else None
+    mode = LOSS_GSPO if cfg.loss == "gspo" else LOSS_GRPO
+
+    stage_events = []
+
+    def step(record=False):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if record else None
+        if record:
+            ev[0].record()
+        lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, cfg.temperature, need_entropy=True)
+        if record:
+            ev[1].record()
+        if train:
+            res = ops.policy_loss(lp, old, adv, mode=mode, cu_seqlens=cu, ref_logprob=ref, entropy=ent,
+                                  loss_mask=mask, diff_clip_ratio=cfg.diff_clip_ratio,
+                                  pos_clip_ratio=cfg.pos_clip_ratio, neg_clip_ratio=cfg.neg_clip_ratio,
+                                  final_clip_ratio=cfg.final_clip_ratio, kl_coef=cfg.kl_coef,
+                                  entropy_coef=cfg.entropy_coef, grad_scale=1.0 / n_tok, want_dloss=False,
+                                  want_upstream=True)
+            if record:
+                ev[2].record()
+            ops.lmhead_backward(hidden, weight, labels, lse, ent, res.g_logprob, res.g_entropy, cfg.temperature,
+                                need_dhidden=True, need_dweight=True, dweight=dweight, accumulate_dweight=False)
+        elif record:
+            ev[2].record()
+        if record:
+            ev[3].record()
+            stage_events.append(ev)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(record=True)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in stage_events) / len(stage_events)
+    loss_ms = sum(e[1].elapsed_time(e[2]) for e in stage_events) / len(stage_events)
+    bwd_ms = sum(e[2].elapsed_time(e[3]) for e in stage_events) / len(stage_events)
+
+    thv = float(T) * cfg.H * cfg.V
+    peak = PEAK_BF16_TFLOPS if cfg.dtype == torch.bfloat16 else PEAK_F32_TFLOPS
+    fwd_tflops = 2.0 * thv / (fwd_ms * 1e-3) / 1e12
+    step_flops = (6.0 if train else 2.0) * thv
+    out = {
+        "metric": "packed tokens/sec, fused logprob+GRPO loss fwd+bwd (Qwen3-8B head); % MFMA peak",
+        "value": T / dt,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if cfg.dtype == torch.bfloat16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: H={cfg.H} V={cfg.V} T={T} packed tokens in {len(samples)} sequences, "
+                               f"{cfg.loss or 'no-grad logprob+entropy'}"
+                               f"{' fwd+bwd (dhidden ' + str(cfg.dtype).split('.')[-1] + ', dW fp32)' if train else ''}",
+                   "temperature": cfg.temperature, "kl_coef": cfg.kl_coef, "entropy_coef": cfg.entropy_coef},
+        "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tflops, "peak": peak,
+                     "unit": "TFLOP/s", "frac": fwd_tflops / peak, "traffic": None,
+                     "algorithmic_flops_per_launch": 2.0 * thv, "avg_launch_ms": fwd_ms},
+        "step_mfma_frac": step_flops / dt / 1e12 / peak,
+        "stage_ms": {"forward": fwd_ms, "loss": loss_ms, "backward": bwd_ms},
+    }
+    if not args.no_unfused and train:
+        try:
+            u_dt = unfused_gpu(cfg, hidden, weight, labels, old, ref, adv, cu, mask, n_tok, max(2, args.steps // 3))
+            out["unfused_torch_gpu"] = {"tokens_per_s": T / u_dt, "ms_per_step": u_dt * 1e3,
+                                        "speedup_fused": u_dt / dt}
+        except Exception as e:  # the unfused path can run out of memory on large configs
+            out["unfused_torch_gpu"] = {"error": str(e)[:200]}
+    if not args.no_cpu_baseline:
+        threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+        tps, reps = cpu_baseline(cfg, args.cpu_rows, threads)
+        out["cpu_baseline"] = {"value": tps, "unit": "tokens/s", "cores": threads, "kind": "port",
+                               "sample": f"{args.cpu_rows} packed rows at full H and V, fp32, fwd"
+                                         f"{'+bwd' if train else ''}, {reps} timed repetitions"}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,200 @@
+// NT-GEMM workgroup tile for gfx950 (CDNA4): C^[BM x BN] = A[BM x K] * B[BN x K]^T,
+// both operands K-contiguous in memory, fp32 accumulation on the matrix cores.
+//
+// One workgroup of WAVES_M x WAVES_N wavefronts (64 lanes each) owns a BM x BN
+// tile.  K is walked in slabs of 128 bytes per row (64 bf16 or 32 fp32
+// elements).  A slab of A (BM rows) and of B (BN rows) is staged in LDS with a
+// padded row stride of 144 bytes, which keeps the 16-byte fragment reads of 16
+// consecutive rows on distinct banks.  Two LDS stages: while the matrix cores
+// work on stage s, the next slab travels HBM/L2 -> registers -> stage s^1.
+//
+// Accumulator layout (v_mfma_f32_32x32x*): for the 32x32 block (mi, ni) of a
+// wave, lane l, register r hold
+//     row (A index) = mi*32 + 8*(r/4) + 4*(l/32) + (r%4)
+//     col (B index) = ni*32 + (l%32)
+// so a lane owns ONE B row per ni and 16 A rows per (mi, ni).  The callers put
+// the dimension they reduce over (vocabulary, for the softmax statistics) on A,
+// which makes that reduction mostly lane-local.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace clgrpo {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kRowBytes = 128;    // K-slab bytes per tile row
+constexpr int kRowStride = 144;   // LDS row stride in bytes (128 + 16 pad)
+constexpr int kChunksPerRow = 8;  // 16-byte chunks per slab row
+
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> { static constexpr int kSlabK = 64; };
+template <> struct Elem<float> { static constexpr int kSlabK = 32; };
+
+// One 32-byte-of-K step for a 32x32 block: a and b each hold 16 bytes per lane.
+template <typename T>
+__device__ __forceinline__ void mma_block(f32x16& acc, const u32x4& a, const u32x4& b);
+
+template <>
+__device__ __forceinline__ void mma_block<__bf16>(f32x16& acc, const u32x4& a, const u32x4& b) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+
+template <>
+__device__ __forceinline__ void mma_block<float>(f32x16& acc, const u32x4& a, const u32x4& b) {
+  // Four K=2 steps; lane half h, element j stands for k = 4h + j in both operands.
+  f32x4 af = __builtin_bit_cast(f32x4, a);
+  f32x4 bf = __builtin_bit_cast(f32x4, b);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[0], bf[0], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[1], bf[1], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[2], bf[2], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[3], bf[3], acc, 0, 0, 0);
+}
+
+// Row of the accumulator register r within a 32x32 block for this lane.
+__device__ __forceinline__ int acc_row(int r, int lane) {
+  return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+}
+
+template <typename T, int BM_, int BN_, int WAVES_M_, int WAVES_N_>
+struct GemmTile {
+  static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = 64 * kWaves;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int MI = WM / 32, NI = WN / 32;
+  static constexpr int kRowsPerPass = kThreads / kChunksPerRow;
+  static constexpr int kPassA = BM / kRowsPerPass, kPassB = BN / kRowsPerPass;
+  static constexpr int kStageBytes = (BM + BN) * kRowStride;
+  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kSlabK = Elem<T>::kSlabK;
+  static_assert(BM % kRowsPerPass == 0 && BN % kRowsPerPass == 0, "tile rows vs threads");
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 blocks");
+
+  // acc[mi][ni] must be zeroed by the caller.  a_base/b_base point at row 0 of
+  // the tile (K offset 0).  Loads go through range-checked buffer descriptors
+  // that cover exactly the a_rows / b_rows valid rows, so rows past them read
+  // as zero and nothing outside the operands is touched.  The row part of an
+  // address always travels in the per-lane offset (the part the hardware range
+  // check is guaranteed to see); only the in-row K offset rides in the scalar
+  // offset.  K must be a multiple of kSlabK and the rows 16-byte aligned.
+  __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const T* a_base, int64_t lda,
+                                             int a_rows, const T* b_base, int64_t ldb, int b_rows,
+                                             int K, char* lds) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave % WAVES_M;
+    const int wn = wave / WAVES_M;
+    const int ld_row = tid >> 3;
+    const int ld_chunk = tid & 7;
+
+    const int lda_b = (int)(lda * (int64_t)sizeof(T));
+    const int ldb_b = (int)(ldb * (int64_t)sizeof(T));
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(a_base), 0, a_rows * lda_b, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(b_base), 0, b_rows * ldb_b, 0x00020000);
+    const int a_voff = ld_row * lda_b + ld_chunk * 16;
+    const int b_voff = ld_row * ldb_b + ld_chunk * 16;
+    const int a_pass = kRowsPerPass * lda_b;
+    const int b_pass = kRowsPerPass * ldb_b;
+
+    const int st_off = ld_row * kRowStride + ld_chunk * 16;
+    const int a_frag_off = (wm * WM + (lane & 31)) * kRowStride + (lane >> 5) * 16;
+    const int b_frag_off = BM * kRowStride + (wn * WN + (lane & 31)) * kRowStride + (lane >> 5) * 16;
+
+    u32x4 ra[kPassA], rb[kPassB];
+    const int nslab = K / kSlabK;
+
+#pragma unroll
+    for (int p = 0; p < kPassA; ++p) ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, 0, 0);
+#pragma unroll
+    for (int p = 0; p < kPassB; ++p) rb[p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, 0, 0);
+#pragma unroll
+    for (int p = 0; p < kPassA; ++p)
+      *reinterpret_cast<u32x4*>(lds + st_off + p * kRowsPerPass * kRowStride) = ra[p];
+#pragma unroll
+    for (int p = 0; p < kPassB; ++p)
+      *reinterpret_cast<u32x4*>(lds + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[p];
+    __syncthreads();
+
+    for (int s = 0; s < nslab; ++s) {
+      char* cur = lds + (s & 1) * kStageBytes;
+      char* nxt = lds + ((s & 1) ^ 1) * kStageBytes;
+      const bool more = (s + 1) < nslab;
+      if (more) {
+        const int koff = (s + 1) * kRowBytes;
+#pragma unroll
+        for (int p = 0; p < kPassA; ++p)
+          ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, koff, 0);
+#pragma unroll
+        for (int p = 0; p < kPassB; ++p)
+          rb[p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, koff, 0);
+      }
+      // Fragments of K-step kk+1 are fetched from LDS before the matrix
+      // instructions of step kk are issued, so the LDS latency hides behind them.
+      u32x4 af[2][MI], bf[2][NI];
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+        af[0][mi] = *reinterpret_cast<const u32x4*>(cur + a_frag_off + mi * 32 * kRowStride);
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+        bf[0][ni] = *reinterpret_cast<const u32x4*>(cur + b_frag_off + ni * 32 * kRowStride);
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        if (kk < 3) {
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi)
+            af[(kk + 1) & 1][mi] =
+                *reinterpret_cast<const u32x4*>(cur + a_frag_off + mi * 32 * kRowStride + (kk + 1) * 32);
+#pragma unroll
+          for (int ni = 0; ni < NI; ++ni)
+            bf[(kk + 1) & 1][ni] =
+                *reinterpret_cast<const u32x4*>(cur + b_frag_off + ni * 32 * kRowStride + (kk + 1) * 32);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of this step's matrix ops
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NI; ++ni) mma_block<T>(acc[mi][ni], af[kk & 1][mi], bf[kk & 1][ni]);
+      }
+      if (more) {
+#pragma unroll
+        for (int p = 0; p < kPassA; ++p)
+          *reinterpret_cast<u32x4*>(nxt + st_off + p * kRowsPerPass * kRowStride) = ra[p];
+#pragma unroll
+        for (int p = 0; p < kPassB; ++p)
+          *reinterpret_cast<u32x4*>(nxt + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[p];
+      }
+      __syncthreads();
+    }
+  }
+};
+
+// Workgroup id -> logical work item so that the workgroups resident on one XCD
+// (hardware deals consecutive ids round-robin over the 8 XCDs) own a contiguous
+// range of logical items and therefore share operand tiles in that XCD's L2.
+// grid must be padded to a multiple of 8; items >= n_items return -1.
+__device__ __forceinline__ int xcd_remap(int bid, int grid) {
+  const int per_xcd = grid >> 3;
+  return (bid & 7) * per_xcd + (bid >> 3);
+}
+
+// Logical item -> (m tile, n tile), walking groups of `gm` m-tiles across all n
+// tiles so neighbours in the logical order share A rows or B rows.
+__device__ __forceinline__ void grouped_tile(int item, int n_m, int n_n, int gm, int& mt, int& nt) {
+  const int per_group = gm * n_n;
+  const int g = item / per_group;
+  const int first_m = g * gm;
+  const int rows = (n_m - first_m) < gm ? (n_m - first_m) : gm;
+  const int in_g = item - g * per_group;
+  mt = first_m + in_g % rows;
+  nt = in_g / rows;
+}
+
+}  // namespace clgrpo

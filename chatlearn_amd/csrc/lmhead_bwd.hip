@@ -1,0 +1,390 @@
+// Backward of the fused lm_head + log-softmax statistics.
+//
+// Per chunk of tokens (the chunk length is set by the workspace the caller gives):
+//   1. dz kernel: recompute a z^T tile [256 vocab x 256 tokens] on the matrix cores
+//      exactly as the forward does, turn it into d(logits) with the stored lse,
+//      and write it in both orientations, dz[token][vocab] and dzT[vocab][token].
+//   2. dhidden[chunk] = dz * W        as an NT GEMM against WT = W^T (built once per call)
+//   3. dW (+)= dzT * hidden[chunk]    as an NT GEMM against hidT = hidden[chunk]^T, fp32 out
+// Every contraction runs through the same K-contiguous MFMA tile (gemm_core.hpp).
+//
+// Algorithmic work: 4*T*H*V flop (dhidden + dW); the z recomputation (2*T*H*V) is overhead.
+#include "common.hpp"
+#include "gemm_core.hpp"
+
+namespace clgrpo {
+
+int validate_head_shape(const char* who, int64_t T, int64_t H, int64_t V, int32_t dtype);
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename T> struct Pack4;
+template <> struct Pack4<float> {
+  typedef float4 type;
+  __device__ static __forceinline__ type make(float a, float b, float c, float d) { return make_float4(a, b, c, d); }
+};
+template <> struct Pack4<__bf16> {
+  typedef uint2 type;
+  __device__ static __forceinline__ type make(float a, float b, float c, float d) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 lo = {(__bf16)a, (__bf16)b};
+    bf16x2 hi = {(__bf16)c, (__bf16)d};
+    return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+  }
+};
+
+struct DzParams {
+  const void* hidden;   // chunk base: [Tc, H]
+  const void* weight;   // [V, H]
+  const int64_t* labels;  // chunk base
+  const float* lse;
+  const float* entropy;   // or nullptr
+  const float* g_lp;
+  const float* g_ent;     // or nullptr
+  int Tc;       // valid tokens in the chunk
+  int ldt;      // dzT row stride = Tc rounded up to 64
+  int H, V;
+  int ldv;      // dz row stride = V rounded up to 64
+  int n_tb, n_vt;
+  float c, inv_temperature;
+  void* dz;     // [Tc][ldv]
+  void* dzT;    // [V][ldt]
+};
+
+template <typename T>
+__global__ __launch_bounds__(512) void lmhead_dz_kernel(DzParams p) {
+  using Tile = GemmTile<T, 256, 256, 2, 4>;
+  constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
+  extern __shared__ __align__(16) char lds[];
+
+  const int item = xcd_remap(blockIdx.x, gridDim.x);
+  if (item >= p.n_tb * p.n_vt) return;
+  int vt, tb;
+  grouped_tile(item, p.n_vt, p.n_tb, 4, vt, tb);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave % 2, wn = wave / 2;
+  const int t0 = tb * 256, v0 = vt * 256;
+  const int b_rows = (p.Tc - t0) < 256 ? (p.Tc - t0) : 256;
+  const int a_rows = (p.V - v0) < 256 ? (p.V - v0) : 256;
+  const T* hidden = static_cast<const T*>(p.hidden) + (int64_t)t0 * p.H;
+  const T* weight = static_cast<const T*>(p.weight) + (int64_t)v0 * p.H;
+
+  // Per-token coefficients.  Tokens past the chunk get zero gradient and a huge lse, so p = 0.
+  int lab[NI], tl[NI];
+  float lse2[NI], lse[NI], glp[NI], gent[NI], ent[NI];
+  bool any_grad = false;
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+    tl[ni] = t0 + wn * WN + ni * 32 + (lane & 31);
+    const bool ok = tl[ni] < p.Tc;
+    lab[ni] = ok ? (int)p.labels[tl[ni]] : -1;
+    lse[ni] = ok ? p.lse[tl[ni]] : 1e30f;
+    lse2[ni] = lse[ni] * kLog2e;
+    glp[ni] = ok ? p.g_lp[tl[ni]] : 0.f;
+    gent[ni] = (ok && p.g_ent) ? p.g_ent[tl[ni]] : 0.f;
+    ent[ni] = (ok && p.g_ent) ? p.entropy[tl[ni]] : 0.f;
+    any_grad |= (glp[ni] != 0.f) | (gent[ni] != 0.f);
+  }
+  // A token block whose upstream gradients are all zero (e.g. prompt-only rows) needs no GEMM.
+  const bool block_live = __syncthreads_or(any_grad);
+
+  f32x16 acc[MI][NI];
+#pragma unroll
+  for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+  if (block_live) Tile::run(acc, weight, p.H, a_rows, hidden, p.H, b_rows, p.H, lds);
+
+  T* dz = static_cast<T*>(p.dz);
+  T* dzT = static_cast<T*>(p.dzT);
+  const float it = p.inv_temperature;
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+    const int rel = lab[ni] - (v0 + wm * WM);
+    const float hot = it * glp[ni];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float d[4];
+        const int row0 = wm * WM + mi * 32 + 8 * q + 4 * (lane >> 5);  // tile row of r = 4q
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float zraw = acc[mi][ni][4 * q + j];
+          const float pr = __builtin_amdgcn_exp2f(fmaf(zraw, p.c, -lse2[ni]));
+          const float logp = fmaf(zraw, it, -lse[ni]);
+          // dz = it * ( glp*(1[v==y] - p) - gent * p * (logp + ent) )
+          float v = -it * pr * fmaf(gent[ni], logp + ent[ni], glp[ni]);
+          if (rel == (row0 - wm * WM) + j) v += hot;
+          if (row0 + j >= a_rows || !block_live) v = 0.f;   // vocabulary padding columns / dead block
+          d[j] = v;
+        }
+        const int v_idx = v0 + row0;
+        if (tl[ni] < p.Tc && v_idx < p.ldv) {
+          typedef typename Pack4<T>::type P4;
+          *reinterpret_cast<P4*>(dz + (int64_t)tl[ni] * p.ldv + v_idx) = Pack4<T>::make(d[0], d[1], d[2], d[3]);
+        }
+        if (tl[ni] < p.ldt) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (v_idx + j < p.V) dzT[(int64_t)(v_idx + j) * p.ldt + tl[ni]] = (T)d[j];
+        }
+      }
+    }
+  }
+}
+
+// C[m][n] (+)= alpha * sum_k A[m][k] B[n][k];  C row-major with leading dimension ldc.
+struct GemmParams {
+  const void* A;
+  const void* B;
+  void* C;
+  int64_t lda, ldb, ldc;
+  int M, N, K;
+  int n_mt, n_nt;
+  int accumulate;
+};
+
+template <typename OutT> __device__ __forceinline__ OutT cvt_out(float v);
+template <> __device__ __forceinline__ float cvt_out<float>(float v) { return v; }
+template <> __device__ __forceinline__ __bf16 cvt_out<__bf16>(float v) { return (__bf16)v; }
+
+template <typename T, typename OutT>
+__global__ __launch_bounds__(512) void gemm_nt_kernel(GemmParams p) {
+  using Tile = GemmTile<T, 256, 256, 2, 4>;
+  constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
+  extern __shared__ __align__(16) char lds[];
+
+  const int item = xcd_remap(blockIdx.x, gridDim.x);
+  if (item >= p.n_mt * p.n_nt) return;
+  int mt, nt;
+  grouped_tile(item, p.n_mt, p.n_nt, 8, mt, nt);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave % 2, wn = wave / 2;
+  const int m0 = mt * 256, n0 = nt * 256;
+  const int a_rows = (p.M - m0) < 256 ? (p.M - m0) : 256;
+  const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
+
+  f32x16 acc[MI][NI];
+#pragma unroll
+  for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+
+  Tile::run(acc, static_cast<const T*>(p.A) + (int64_t)m0 * p.lda, p.lda, a_rows,
+            static_cast<const T*>(p.B) + (int64_t)n0 * p.ldb, p.ldb, b_rows, p.K, lds);
+
+  OutT* C = static_cast<OutT*>(p.C);
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+    const int col = wn * WN + ni * 32 + (lane & 31);
+    if (col >= b_rows) continue;
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = wm * WM + mi * 32 + acc_row(r, lane);
+        if (row < a_rows) {
+          OutT* dst = C + (int64_t)(m0 + row) * p.ldc + (n0 + col);
+          float v = acc[mi][ni][r];
+          if (p.accumulate) v += (float)*dst;
+          *dst = cvt_out<OutT>(v);
+        }
+      }
+  }
+}
+
+// dst[c][r] = src[r][c] for r < R, c < C; dst[c][r] = 0 for R <= r < ld_dst.  64x64 tiles.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_pad_kernel(const T* __restrict__ src, int64_t ld_src,
+                                                            T* __restrict__ dst, int64_t ld_dst, int R, int C) {
+  __shared__ T tile[64][65];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i, c = c0 + tx;
+    tile[i][tx] = (r < R && c < C) ? src[(int64_t)r * ld_src + c] : (T)0.f;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int c = c0 + i, r = r0 + tx;
+    if (c < C && r < ld_dst) dst[(int64_t)c * ld_dst + r] = tile[tx][i];
+  }
+}
+
+struct BwdPlan {
+  int64_t ldv;        // dz / WT row stride
+  int64_t chunk;      // tokens per chunk (multiple of 256 unless >= T)
+  int64_t ldt;        // dzT / hidT row stride for a full chunk
+  size_t off_wt, off_hidt, off_dz, off_dzt, total;
+};
+
+static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chunk_tokens) {
+  BwdPlan pl;
+  pl.ldv = round_up64(V, 64);
+  int64_t chunk = (chunk_tokens <= 0 || chunk_tokens >= T) ? T : round_up64(chunk_tokens, 256);
+  if (chunk > T) chunk = T;
+  pl.chunk = chunk;
+  pl.ldt = round_up64(chunk, 64);
+  size_t off = 0;
+  pl.off_wt = off;   off += align_up((size_t)H * pl.ldv * es, 256);
+  pl.off_hidt = off; off += align_up((size_t)H * pl.ldt * es, 256);
+  pl.off_dz = off;   off += align_up((size_t)chunk * pl.ldv * es, 256);
+  pl.off_dzt = off;  off += align_up((size_t)V * pl.ldt * es, 256);
+  pl.total = off;
+  return pl;
+}
+
+// Largest chunk (multiple of 256, or T itself) whose plan fits into `bytes`; 0 if none does.
+static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, size_t bytes) {
+  if (bwd_plan(T, H, V, es, T).total <= bytes) return T;
+  int64_t lo = 0, hi = T / 256;   // in units of 256 tokens
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) / 2;
+    if (bwd_plan(T, H, V, es, mid * 256).total <= bytes) lo = mid; else hi = mid - 1;
+  }
+  return lo * 256;
+}
+
+template <typename T>
+static int set_lds_attr(const void* fn, const char* name) {
+  using Tile = GemmTile<T, 256, 256, 2, 4>;
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
+  if (e != hipSuccess) return fail(CLGRPO_ELAUNCH, "%s: LDS attribute: %s", name, hipGetErrorString(e));
+  return CLGRPO_OK;
+}
+
+template <typename T, typename OutT>
+static int launch_gemm(const void* A, int64_t lda, int M, const void* B, int64_t ldb, int N, int K, void* C,
+                       int64_t ldc, int accumulate, hipStream_t stream) {
+  using Tile = GemmTile<T, 256, 256, 2, 4>;
+  static bool attr = false;
+  if (!attr) {
+    int rc = set_lds_attr<T>(reinterpret_cast<const void*>(&gemm_nt_kernel<T, OutT>), "gemm_nt_kernel");
+    if (rc) return rc;
+    attr = true;
+  }
+  GemmParams g;
+  g.A = A; g.B = B; g.C = C; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.M = M; g.N = N; g.K = K;
+  g.n_mt = (M + 255) / 256; g.n_nt = (N + 255) / 256;
+  g.accumulate = accumulate;
+  int grid = (g.n_mt * g.n_nt + 7) / 8 * 8;
+  hipLaunchKernelGGL((gemm_nt_kernel<T, OutT>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, g);
+  return check_launch("gemm_nt_kernel");
+}
+
+template <typename T>
+static int launch_transpose(const T* src, int64_t ld_src, T* dst, int64_t ld_dst, int R, int C, hipStream_t stream) {
+  dim3 grid((C + 63) / 64, (int)((ld_dst + 63) / 64));
+  hipLaunchKernelGGL(transpose_pad_kernel<T>, grid, dim3(256), 0, stream, src, ld_src, dst, ld_dst, R, C);
+  return check_launch("transpose_pad_kernel");
+}
+
+template <typename T>
+static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream) {
+  using Tile = GemmTile<T, 256, 256, 2, 4>;
+  const int64_t T_ = a->T, H = a->H, V = a->V;
+  const int64_t chunk = chunk_for_workspace(T_, H, V, sizeof(T), a->workspace_bytes);
+  if (chunk <= 0)
+    return fail(CLGRPO_EWORKSPACE, "clgrpo_lmhead_bwd: workspace %zu bytes cannot hold a 256-token chunk (%zu needed)",
+                a->workspace_bytes, bwd_plan(T_, H, V, sizeof(T), 256).total);
+  const BwdPlan pl = bwd_plan(T_, H, V, sizeof(T), chunk);
+  char* ws = static_cast<char*>(a->workspace);
+  T* wt = reinterpret_cast<T*>(ws + pl.off_wt);
+  T* hidt = reinterpret_cast<T*>(ws + pl.off_hidt);
+  T* dz = reinterpret_cast<T*>(ws + pl.off_dz);
+  T* dzt = reinterpret_cast<T*>(ws + pl.off_dzt);
+  const T* hidden = static_cast<const T*>(a->hidden);
+  const T* weight = static_cast<const T*>(a->weight);
+
+  static bool attr = false;
+  if (!attr) {
+    int rc = set_lds_attr<T>(reinterpret_cast<const void*>(&lmhead_dz_kernel<T>), "lmhead_dz_kernel");
+    if (rc) return rc;
+    attr = true;
+  }
+  int rc;
+  if (a->dhidden) {
+    // WT[h][v] = W[v][h], zero for V <= v < ldv
+    rc = launch_transpose<T>(weight, H, wt, pl.ldv, (int)V, (int)H, stream);
+    if (rc) return rc;
+  }
+  for (int64_t c0 = 0; c0 < T_; c0 += chunk) {
+    const int64_t tc = (T_ - c0) < chunk ? (T_ - c0) : chunk;
+    const int64_t ldt = round_up64(tc, 64);
+    DzParams d;
+    d.hidden = hidden + c0 * H;
+    d.weight = weight;
+    d.labels = a->labels + c0;
+    d.lse = a->lse + c0;
+    d.entropy = a->g_entropy ? a->entropy + c0 : nullptr;
+    d.g_lp = a->g_logprob + c0;
+    d.g_ent = a->g_entropy ? a->g_entropy + c0 : nullptr;
+    d.Tc = (int)tc;
+    d.ldt = (int)ldt;
+    d.H = (int)H;
+    d.V = (int)V;
+    d.ldv = (int)pl.ldv;
+    d.n_tb = (int)((ldt + 255) / 256);
+    d.n_vt = (int)((V + 255) / 256);
+    d.c = a->inv_temperature * kLog2e;
+    d.inv_temperature = a->inv_temperature;
+    d.dz = dz;
+    d.dzT = dzt;
+    int grid = (d.n_tb * d.n_vt + 7) / 8 * 8;
+    hipLaunchKernelGGL(lmhead_dz_kernel<T>, dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, d);
+    rc = check_launch("lmhead_dz_kernel");
+    if (rc) return rc;
+    if (a->dhidden) {
+      // dhidden[chunk][h] = sum_v dz[t][v] WT[h][v]
+      rc = launch_gemm<T, T>(dz, pl.ldv, (int)tc, wt, pl.ldv, (int)H, (int)pl.ldv,
+                             static_cast<T*>(a->dhidden) + c0 * H, H, 0, stream);
+      if (rc) return rc;
+    }
+    if (a->dweight) {
+      // hidT[h][t] = hidden[c0 + t][h], zero for tc <= t < ldt;  dW[v][h] (+)= sum_t dzT[v][t] hidT[h][t]
+      rc = launch_transpose<T>(hidden + c0 * H, H, hidt, ldt, (int)tc, (int)H, stream);
+      if (rc) return rc;
+      rc = launch_gemm<T, float>(dzt, ldt, (int)V, hidt, ldt, (int)H, (int)ldt, a->dweight, H,
+                                 (a->accumulate_dweight || c0 > 0) ? 1 : 0, stream);
+      if (rc) return rc;
+    }
+  }
+  return CLGRPO_OK;
+}
+
+}  // namespace clgrpo
+
+using namespace clgrpo;
+
+extern "C" size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype,
+                                                    int64_t chunk_tokens) {
+  if (T <= 0 || H <= 0 || V <= 0 || (dtype != CLGRPO_BF16 && dtype != CLGRPO_F32)) return 0;
+  return bwd_plan(T, H, V, dtype_bytes(dtype), chunk_tokens).total;
+}
+
+extern "C" int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream) {
+  CLGRPO_REQUIRE_PTR(a, "args");
+  int rc = validate_head_shape("clgrpo_lmhead_bwd", a->T, a->H, a->V, a->dtype);
+  if (rc) return rc;
+  CLGRPO_REQUIRE_PTR(a->hidden, "hidden");
+  CLGRPO_REQUIRE_PTR(a->weight, "weight");
+  CLGRPO_REQUIRE_PTR(a->labels, "labels");
+  CLGRPO_REQUIRE_PTR(a->lse, "lse");
+  CLGRPO_REQUIRE_PTR(a->g_logprob, "g_logprob");
+  if (a->g_entropy != nullptr) CLGRPO_REQUIRE_PTR(a->entropy, "entropy");
+  if (a->dhidden == nullptr && a->dweight == nullptr)
+    return fail(CLGRPO_ENULL, "clgrpo_lmhead_bwd: both dhidden and dweight are NULL");
+  if (!(a->inv_temperature > 0.f)) return fail(CLGRPO_EINVAL, "clgrpo_lmhead_bwd: inv_temperature must be > 0");
+  CLGRPO_REQUIRE_PTR(a->workspace, "workspace");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return a->dtype == CLGRPO_BF16 ? run_bwd<__bf16>(a, s) : run_bwd<float>(a, s);
+}

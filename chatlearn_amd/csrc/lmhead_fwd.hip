@@ -1,0 +1,316 @@
+// Fused lm_head projection + online log-softmax statistics (forward).
+//
+// z^T tile [256 vocab x 256 tokens] = W tile * hidden tile^T on the matrix cores;
+// the vocabulary runs along the accumulator registers, the tokens along the
+// lanes, so each lane keeps a running (max, sum e^{z-max}, sum e^{z-max} z,
+// target logit) for its own tokens across all vocabulary tiles of its split.
+// A workgroup owns one block of 256 tokens and one contiguous range of
+// vocabulary tiles ("split"); a second small kernel merges the splits with an
+// exact rescale and writes logprob / entropy / rowmax / lse.  Logits never go
+// to memory.
+//
+// Algorithmic work: 2*T*H*V flop; bytes 2*T*H + 2*V*H (bf16) + 16*T.
+#include "common.hpp"
+#include "gemm_core.hpp"
+
+namespace clgrpo {
+
+constexpr int kFwdBM = 256, kFwdBN = 256;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct FwdParams {
+  const void* hidden;
+  const void* weight;
+  const int64_t* labels;
+  int T, H, V;
+  int n_tb, n_split, tiles_per_split, n_vt;
+  float c;  // inv_temperature * log2(e)
+  float4* part;  // [n_split][T]: (max raw, sum 2^{(z-max) c}, sum 2^{(z-max) c} z raw, target raw)
+};
+
+__device__ __forceinline__ void merge_state(float& m, float& s, float& u, float om, float os,
+                                            float ou, float c) {
+  const float nm = fmaxf(m, om);
+  const float a = (m == nm) ? 1.f : exp2f((m - nm) * c);
+  const float b = (om == nm) ? 1.f : exp2f((om - nm) * c);
+  s = s * a + os * b;
+  u = u * a + ou * b;
+  m = nm;
+}
+
+template <typename T>
+__global__ __launch_bounds__(512) void lmhead_fwd_kernel(FwdParams p) {
+  using Tile = GemmTile<T, kFwdBM, kFwdBN, 2, 4>;
+  constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
+  extern __shared__ __align__(16) char lds[];
+
+  const int item = xcd_remap(blockIdx.x, gridDim.x);
+  if (item >= p.n_tb * p.n_split) return;
+  int vs, tb;
+  grouped_tile(item, p.n_split, p.n_tb, 4, vs, tb);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave % 2, wn = wave / 2;
+  const int t0 = tb * kFwdBN;
+  const int b_rows = (p.T - t0) < kFwdBN ? (p.T - t0) : kFwdBN;
+  const T* hidden = static_cast<const T*>(p.hidden) + (int64_t)t0 * p.H;
+  const T* weight = static_cast<const T*>(p.weight);
+  const float c = p.c;
+
+  int lab[NI];
+  float m[NI], s[NI], u[NI], zt[NI];
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+    const int tok = t0 + wn * WN + ni * 32 + (lane & 31);
+    lab[ni] = (p.labels != nullptr && tok < p.T) ? (int)p.labels[tok] : -1;
+    m[ni] = -INFINITY;
+    s[ni] = 0.f;
+    u[ni] = 0.f;
+    zt[ni] = 0.f;
+  }
+
+  const int vt_begin = vs * p.tiles_per_split;
+  const int vt_end = (vt_begin + p.tiles_per_split) < p.n_vt ? (vt_begin + p.tiles_per_split) : p.n_vt;
+  for (int vt = vt_begin; vt < vt_end; ++vt) {
+    const int v0 = vt * kFwdBM;
+    const int a_rows = (p.V - v0) < kFwdBM ? (p.V - v0) : kFwdBM;
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+
+    Tile::run(acc, weight + (int64_t)v0 * p.H, p.H, a_rows, hidden, p.H, b_rows, p.H, lds);
+
+    if (a_rows == kFwdBM) {
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+        float tmax = acc[0][ni][0];
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, acc[mi][ni][r]);
+        const float nm = fmaxf(m[ni], tmax);
+        const float scale = exp2f((m[ni] - nm) * c);  // m = -inf on the first tile -> 0
+        const float nb = -nm * c;
+        float ls = 0.f, lu = 0.f;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float v = acc[mi][ni][r];
+            const float e = __builtin_amdgcn_exp2f(fmaf(v, c, nb));
+            ls += e;
+            lu = fmaf(e, v, lu);
+          }
+        s[ni] = fmaf(s[ni], scale, ls);
+        u[ni] = fmaf(u[ni], scale, lu);
+        m[ni] = nm;
+      }
+    } else {
+      // Last, partial vocabulary tile: rows >= a_rows are clamped duplicates and must not count.
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int row = wm * WM + mi * 32 + acc_row(r, lane);
+            if (row < a_rows) tmax = fmaxf(tmax, acc[mi][ni][r]);
+          }
+        const float nm = fmaxf(m[ni], tmax);
+        if (nm == -INFINITY) continue;  // this lane has seen no valid row yet
+        const float scale = exp2f((m[ni] - nm) * c);
+        const float nb = -nm * c;
+        float ls = 0.f, lu = 0.f;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int row = wm * WM + mi * 32 + acc_row(r, lane);
+            if (row < a_rows) {
+              const float v = acc[mi][ni][r];
+              const float e = __builtin_amdgcn_exp2f(fmaf(v, c, nb));
+              ls += e;
+              lu = fmaf(e, v, lu);
+            }
+          }
+        s[ni] = fmaf(s[ni], scale, ls);
+        u[ni] = fmaf(u[ni], scale, lu);
+        m[ni] = nm;
+      }
+    }
+
+    // Target logit: only the wave whose 128 vocabulary rows hold the label looks for it.
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+      const int rel = lab[ni] - (v0 + wm * WM);
+      const bool in = (unsigned)rel < (unsigned)WM && (lab[ni] < p.V);
+      if (__any(in)) {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (rel == mi * 32 + acc_row(r, lane)) zt[ni] = acc[mi][ni][r];
+      }
+    }
+  }
+
+  // Merge the two lane halves (same tokens, different vocabulary rows).
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+    const float om = __shfl_xor(m[ni], 32);
+    const float os = __shfl_xor(s[ni], 32);
+    const float ou = __shfl_xor(u[ni], 32);
+    const float oz = __shfl_xor(zt[ni], 32);
+    merge_state(m[ni], s[ni], u[ni], om, os, ou, c);
+    zt[ni] += oz;
+  }
+  // Merge the two waves that share these tokens (wm = 0, 1) through LDS.
+  float4* xch = reinterpret_cast<float4*>(lds);
+  if (wm == 1 && lane < 32) {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+      xch[wn * WN + ni * 32 + lane] = make_float4(m[ni], s[ni], u[ni], zt[ni]);
+  }
+  __syncthreads();
+  if (wm == 0 && lane < 32) {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+      const float4 o = xch[wn * WN + ni * 32 + lane];
+      merge_state(m[ni], s[ni], u[ni], o.x, o.y, o.z, c);
+      zt[ni] += o.w;
+      const int tok = t0 + wn * WN + ni * 32 + lane;
+      if (tok < p.T) p.part[(int64_t)vs * p.T + tok] = make_float4(m[ni], s[ni], u[ni], zt[ni]);
+    }
+  }
+}
+
+struct FinalizeParams {
+  const float4* part;
+  const int64_t* labels;
+  int T, V, n_split;
+  float c, inv_temperature;
+  float* logprob;
+  float* entropy;
+  float* rowmax;
+  float* lse;
+};
+
+__global__ void lmhead_fwd_finalize_kernel(FinalizeParams p) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= p.T) return;
+  float m = -INFINITY, s = 0.f, u = 0.f, zt = 0.f;
+  for (int k = 0; k < p.n_split; ++k) {
+    const float4 o = p.part[(int64_t)k * p.T + t];
+    merge_state(m, s, u, o.x, o.y, o.z, p.c);
+    zt += o.w;
+  }
+  const float mx = m * p.inv_temperature;
+  const float lse = mx + logf(s);
+  p.lse[t] = lse;
+  if (p.rowmax) p.rowmax[t] = mx;
+  if (p.entropy) p.entropy[t] = lse - p.inv_temperature * u / s;
+  if (p.logprob) {
+    const int64_t lab = p.labels[t];
+    // A label outside [0, V) has no logit; NaN marks it instead of a silent wrong number.
+    p.logprob[t] = (lab >= 0 && lab < p.V) ? (zt * p.inv_temperature - lse) : NAN;
+  }
+}
+
+static void fwd_plan(int64_t T, int64_t V, int& n_tb, int& n_vt, int& n_split, int& tiles_per_split) {
+  n_tb = (int)((T + kFwdBN - 1) / kFwdBN);
+  n_vt = (int)((V + kFwdBM - 1) / kFwdBM);
+  int cus = 256;
+  int want = cus / n_tb;
+  if (want < 4) want = 4;
+  if (want > n_vt) want = n_vt;
+  tiles_per_split = (n_vt + want - 1) / want;
+  n_split = (n_vt + tiles_per_split - 1) / tiles_per_split;
+}
+
+template <typename T>
+static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream) {
+  using Tile = GemmTile<T, kFwdBM, kFwdBN, 2, 4>;
+  FwdParams p;
+  p.hidden = a->hidden;
+  p.weight = a->weight;
+  p.labels = a->labels;
+  p.T = (int)a->T;
+  p.H = (int)a->H;
+  p.V = (int)a->V;
+  fwd_plan(a->T, a->V, p.n_tb, p.n_vt, p.n_split, p.tiles_per_split);
+  p.c = a->inv_temperature * kLog2e;
+  p.part = static_cast<float4*>(a->workspace);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&lmhead_fwd_kernel<T>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
+    if (e != hipSuccess) return fail(CLGRPO_ELAUNCH, "lmhead_fwd: LDS attribute: %s", hipGetErrorString(e));
+    attr_set = true;
+  }
+  int grid = p.n_tb * p.n_split;
+  grid = (grid + 7) / 8 * 8;
+  hipLaunchKernelGGL(lmhead_fwd_kernel<T>, dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, p);
+  int rc = check_launch("lmhead_fwd_kernel");
+  if (rc) return rc;
+  FinalizeParams f;
+  f.part = p.part;
+  f.labels = a->labels;
+  f.T = p.T;
+  f.V = p.V;
+  f.n_split = p.n_split;
+  f.c = p.c;
+  f.inv_temperature = a->inv_temperature;
+  f.logprob = a->labels ? a->logprob : nullptr;
+  f.entropy = a->entropy;
+  f.rowmax = a->rowmax;
+  f.lse = a->lse;
+  hipLaunchKernelGGL(lmhead_fwd_finalize_kernel, dim3((p.T + 255) / 256), dim3(256), 0, stream, f);
+  return check_launch("lmhead_fwd_finalize_kernel");
+}
+
+int validate_head_shape(const char* who, int64_t T, int64_t H, int64_t V, int32_t dtype) {
+  if (dtype != CLGRPO_BF16 && dtype != CLGRPO_F32) return fail(CLGRPO_EDTYPE, "%s: dtype %d unsupported", who, dtype);
+  if (T <= 0 || H <= 0 || V <= 0) return fail(CLGRPO_EINVAL, "%s: T, H, V must be positive (got %lld, %lld, %lld)", who,
+                                             (long long)T, (long long)H, (long long)V);
+  const int slab = dtype == CLGRPO_BF16 ? 64 : 32;
+  if (H % slab != 0) return fail(CLGRPO_ESHAPE, "%s: H=%lld must be a multiple of %d", who, (long long)H, slab);
+  if (T >= (1LL << 30) || V >= (1LL << 30) || H >= (1LL << 24)) return fail(CLGRPO_ESHAPE, "%s: size too large", who);
+  return CLGRPO_OK;
+}
+
+}  // namespace clgrpo
+
+using namespace clgrpo;
+
+extern "C" size_t clgrpo_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype) {
+  (void)H;
+  (void)dtype;
+  if (T <= 0 || V <= 0) return 0;
+  int n_tb, n_vt, n_split, tps;
+  fwd_plan(T, V, n_tb, n_vt, n_split, tps);
+  return (size_t)n_split * (size_t)T * sizeof(float4);
+}
+
+extern "C" int clgrpo_lmhead_fwd(const clgrpo_lmhead_fwd_args* a, void* stream) {
+  CLGRPO_REQUIRE_PTR(a, "args");
+  int rc = validate_head_shape("clgrpo_lmhead_fwd", a->T, a->H, a->V, a->dtype);
+  if (rc) return rc;
+  CLGRPO_REQUIRE_PTR(a->hidden, "hidden");
+  CLGRPO_REQUIRE_PTR(a->weight, "weight");
+  CLGRPO_REQUIRE_PTR(a->lse, "lse");
+  if (a->labels != nullptr) CLGRPO_REQUIRE_PTR(a->logprob, "logprob");
+  if (!(a->inv_temperature > 0.f)) return fail(CLGRPO_EINVAL, "clgrpo_lmhead_fwd: inv_temperature must be > 0");
+  CLGRPO_REQUIRE_PTR(a->workspace, "workspace");
+  const size_t need = clgrpo_lmhead_fwd_workspace_bytes(a->T, a->H, a->V, a->dtype);
+  if (a->workspace_bytes < need)
+    return fail(CLGRPO_EWORKSPACE, "clgrpo_lmhead_fwd: workspace %zu < %zu bytes", a->workspace_bytes, need);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return a->dtype == CLGRPO_BF16 ? launch_fwd<__bf16>(a, s) : launch_fwd<float>(a, s);
+}

@@ -1,0 +1,370 @@
+"""Torch-tensor front end of the C ABI: allocates outputs / workspaces with torch
+(device memory and streams are all torch is used for) and calls libclgrpo.so.
+
+Every function here requires device tensors and the built library; nothing
+falls back to torch arithmetic.
+"""
+import ctypes as C
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import BF16, F32, F64, LOSS_GRPO, LOSS_GSPO
+
+DEFAULT_BWD_WORKSPACE_BYTES = 24 << 30
+
+
+def _dtype_enum(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return BF16
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.float64:
+        return F64
+    raise TypeError(f"unsupported dtype {t.dtype}")
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (got {t.device}); this package has no CPU path")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+# --------------------------------------------------------------------------- fused lm_head
+
+def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[torch.Tensor],
+                   temperature: float = 1.0, need_entropy: bool = True
+                   ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], torch.Tensor, torch.Tensor]:
+    """(logprob, entropy, rowmax, lse), each fp32 [T]; logits are never materialised."""
+    hidden = _dev(hidden, "hidden")
+    weight = _dev(weight, "weight", hidden.dtype)
+    if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
+        raise ValueError(f"hidden [T,H] / weight [V,H] expected, got {tuple(hidden.shape)} / {tuple(weight.shape)}")
+    T, H = hidden.shape
+    V = weight.shape[0]
+    if labels is not None:
+        labels = _dev(labels, "labels", torch.int64)
+        if labels.numel() != T:
+            raise ValueError(f"labels must have {T} elements, got {labels.numel()}")
+    dt = _dtype_enum(hidden)
+    f = dict(dtype=torch.float32, device=hidden.device)
+    lse = torch.empty(T, **f)
+    rowmax = torch.empty(T, **f)
+    logprob = torch.empty(T, **f) if labels is not None else None
+    entropy = torch.empty(T, **f) if need_entropy else None
+    if T == 0:
+        return logprob, entropy, rowmax, lse
+    ws_bytes = _lib.lib().clgrpo_lmhead_fwd_workspace_bytes(T, H, V, dt)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=hidden.device)
+    a = _lib.LmheadFwdArgs(_ptr(hidden), _ptr(weight), _ptr(labels), T, H, V, dt, 1.0 / float(temperature),
+                           _ptr(logprob), _ptr(entropy), _ptr(rowmax), _ptr(lse), _ptr(ws), ws.numel())
+    _lib.call("clgrpo_lmhead_fwd", a, _stream(hidden))
+    return logprob, entropy, rowmax, lse
+
+
+def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=None, temperature=1.0,
+                    need_dhidden=True, need_dweight=True, dweight: Optional[torch.Tensor] = None,
+                    accumulate_dweight=False, chunk_tokens: Optional[int] = None,
+                    max_workspace_bytes: int = DEFAULT_BWD_WORKSPACE_BYTES):
+    """(dhidden [T,H] in hidden's dtype, dweight [V,H] fp32).  ``dweight`` may be a caller
+    buffer (e.g. the fp32 main-grad) that is overwritten or, with ``accumulate_dweight``, added to."""
+    hidden = _dev(hidden, "hidden")
+    weight = _dev(weight, "weight", hidden.dtype)
+    labels = _dev(labels, "labels", torch.int64)
+    lse = _dev(lse, "lse", torch.float32)
+    g_logprob = _dev(g_logprob, "g_logprob", torch.float32)
+    T, H = hidden.shape
+    V = weight.shape[0]
+    for name, t in (("labels", labels), ("lse", lse), ("g_logprob", g_logprob)):
+        if t.numel() != T:
+            raise ValueError(f"{name} must have {T} elements, got {t.numel()}")
+    if g_entropy is not None:
+        g_entropy = _dev(g_entropy, "g_entropy", torch.float32)
+        entropy = _dev(entropy, "entropy", torch.float32)
+        if g_entropy.numel() != T or entropy.numel() != T:
+            raise ValueError("g_entropy / entropy must have T elements")
+    dt = _dtype_enum(hidden)
+    dhidden = torch.empty_like(hidden) if need_dhidden else None
+    if need_dweight:
+        if dweight is None:
+            dweight = torch.empty(V, H, dtype=torch.float32, device=hidden.device)
+            accumulate_dweight = False
+        else:
+            dweight = _dev(dweight, "dweight", torch.float32)
+            if tuple(dweight.shape) != (V, H) or not dweight.is_contiguous():
+                raise ValueError("dweight must be a contiguous fp32 [V,H] tensor")
+    else:
+        dweight = None
+    if T == 0:
+        if dweight is not None and not accumulate_dweight:
+            dweight.zero_()
+        return dhidden, dweight
+    L = _lib.lib()
+    if chunk_tokens is None:
+        chunk_tokens = T
+        while chunk_tokens > 256 and L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens) > max_workspace_bytes:
+            chunk_tokens = max(256, (chunk_tokens // 2 + 255) // 256 * 256)
+    ws_bytes = L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hidden.device)
+    a = _lib.LmheadBwdArgs(_ptr(hidden), _ptr(weight), _ptr(labels), _ptr(lse), _ptr(entropy), _ptr(g_logprob),
+                           _ptr(g_entropy), T, H, V, dt, 1.0 / float(temperature), _ptr(dhidden), _ptr(dweight),
+                           1 if accumulate_dweight else 0, _ptr(ws), ws.numel())
+    _lib.call("clgrpo_lmhead_bwd", a, _stream(hidden))
+    return dhidden, dweight
+
+
+# --------------------------------------------------------------------------- stats from logits
+
+def softmax_stats(logits2d: torch.Tensor, labels: Optional[torch.Tensor], need_entropy=True, need_logprob=True):
+    """(logprob, entropy, lse) fp32 [R] from materialised [R,V] logits (last dim contiguous)."""
+    if logits2d.dim() != 2:
+        raise ValueError("logits2d must be [R,V]")
+    if not logits2d.is_cuda:
+        raise RuntimeError("logits must live on the GPU; this package has no CPU path")
+    if logits2d.stride(1) != 1:
+        logits2d = logits2d.contiguous()
+    R, V = logits2d.shape
+    ld = logits2d.stride(0) if R > 1 else V
+    dt = _dtype_enum(logits2d)
+    f = dict(dtype=torch.float32, device=logits2d.device)
+    need_logprob = need_logprob and labels is not None
+    if need_logprob:
+        labels = _dev(labels, "labels", torch.int64)
+    lp = torch.empty(R, **f) if need_logprob else None
+    ent = torch.empty(R, **f) if need_entropy else None
+    lse = torch.empty(R, **f)
+    a = _lib.SoftmaxStatsArgs(_ptr(logits2d), _ptr(labels) if need_logprob else None, R, V, ld, dt,
+                              _ptr(lp), _ptr(ent), _ptr(lse))
+    _lib.call("clgrpo_softmax_stats", a, _stream(logits2d))
+    return lp, ent, lse
+
+
+def softmax_stats_backward(logits2d, labels, g_logprob, g_entropy):
+    if not logits2d.is_cuda:
+        raise RuntimeError("logits must live on the GPU; this package has no CPU path")
+    if logits2d.stride(1) != 1:
+        logits2d = logits2d.contiguous()
+    R, V = logits2d.shape
+    ld = logits2d.stride(0) if R > 1 else V
+    out = torch.empty(R, V, dtype=logits2d.dtype, device=logits2d.device)
+    if g_logprob is not None:
+        g_logprob = _dev(g_logprob, "g_logprob", torch.float32)
+        labels = _dev(labels, "labels", torch.int64)
+    if g_entropy is not None:
+        g_entropy = _dev(g_entropy, "g_entropy", torch.float32)
+    a = _lib.SoftmaxStatsBwdArgs(_ptr(logits2d), _ptr(labels) if g_logprob is not None else None, _ptr(g_logprob),
+                                 _ptr(g_entropy), R, V, ld, _dtype_enum(logits2d), _ptr(out))
+    _lib.call("clgrpo_softmax_stats_bwd", a, _stream(logits2d))
+    return out
+
+
+# --------------------------------------------------------------------------- policy loss
+
+class PolicyLossResult:
+    """Outputs of one clgrpo_policy_loss launch (device tensors; ``sums``/``flags`` not yet synced)."""
+    __slots__ = ("loss", "dloss", "kl", "is_positive_clipped", "is_negative_clipped", "is_clipped",
+                 "g_logprob", "g_entropy", "sums", "flags")
+
+    def raise_on_flags(self):
+        """Same assertions, same messages, as the reference raises (one host sync)."""
+        fl = int(self.flags.item())
+        assert not fl & 1, "pg loss is nan"
+        assert not fl & 2, "kl loss ratio has inf values"
+        assert not fl & 4, "kl loss ratio has nan values"
+
+
+def policy_loss(logprob, old_logprob, advantages, *, mode=LOSS_GRPO, cu_seqlens=None, ref_logprob=None,
+                entropy=None, loss_mask=None, diff_clip_ratio=10, pos_clip_ratio=0.2, neg_clip_ratio=0.2,
+                final_clip_ratio=3.0, kl_coef=0.0, entropy_coef=0.0, grad_scale=1.0, want_dloss=True,
+                want_kl=None, want_flags3=False, want_upstream=False) -> PolicyLossResult:
+    """logprob/old/ref/entropy fp32, either [B,S] (padded) or flat [n] with ``cu_seqlens`` int32 [B+1];
+    ``advantages`` a device tensor [B], fp32 or fp64 (sets the dtype of the loss)."""
+    logprob = _dev(logprob, "logprob", torch.float32)
+    old_logprob = _dev(old_logprob, "old_logprob", torch.float32)
+    advantages = _dev(advantages, "advantages")
+    cdt = _dtype_enum(advantages)
+    if cdt not in (F32, F64):
+        raise TypeError("advantages must be fp32 or fp64")
+    n = logprob.numel()
+    if old_logprob.numel() != n:
+        raise ValueError("old_logprob and logprob differ in size")
+    if cu_seqlens is not None:
+        cu_seqlens = _dev(cu_seqlens, "cu_seqlens", torch.int32)
+        B, S = cu_seqlens.numel() - 1, 0
+    else:
+        if logprob.dim() != 2:
+            raise ValueError("padded layout needs [B,S] tensors (or pass cu_seqlens)")
+        B, S = logprob.shape
+    if advantages.numel() != B:
+        raise ValueError(f"advantages must have {B} elements, got {advantages.numel()}")
+    dev = logprob.device
+
+    def opt(t, name, dtype):
+        if t is None:
+            return None
+        t = _dev(t, name, dtype)
+        if t.numel() != n:
+            raise ValueError(f"{name} must have {n} elements")
+        return t
+
+    ref_logprob = opt(ref_logprob, "ref_logprob", torch.float32)
+    entropy = opt(entropy, "entropy", torch.float32)
+    if loss_mask is not None and loss_mask.dtype != torch.int32:
+        loss_mask = loss_mask.to(torch.int32)
+    loss_mask = opt(loss_mask, "loss_mask", torch.int32)
+    if want_kl is None:
+        want_kl = ref_logprob is not None
+    r = PolicyLossResult()
+    r.loss = torch.empty(logprob.shape, dtype=advantages.dtype, device=dev)
+    r.dloss = torch.empty(logprob.shape, dtype=advantages.dtype, device=dev) if want_dloss else None
+    r.kl = torch.empty(logprob.shape, dtype=torch.float32, device=dev) if want_kl else None
+    mk = lambda: torch.empty(logprob.shape, dtype=torch.bool, device=dev)
+    r.is_positive_clipped, r.is_negative_clipped, r.is_clipped = (mk(), mk(), mk()) if want_flags3 else (None, None, None)
+    r.g_logprob = torch.empty(logprob.shape, dtype=torch.float32, device=dev) if want_upstream else None
+    r.g_entropy = (torch.empty(logprob.shape, dtype=torch.float32, device=dev)
+                   if (want_upstream and entropy_coef > 0) else None)
+    r.sums = torch.empty(8, dtype=torch.float64, device=dev)
+    r.flags = torch.empty(1, dtype=torch.int32, device=dev)
+    if n == 0:
+        r.sums.zero_()
+        r.flags.zero_()
+        return r
+    ws_bytes = _lib.lib().clgrpo_policy_loss_workspace_bytes(n, B)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    a = _lib.PolicyLossArgs(mode, cdt, n, B, S, _ptr(cu_seqlens), _ptr(logprob), _ptr(old_logprob), _ptr(ref_logprob),
+                            _ptr(entropy), _ptr(loss_mask), _ptr(advantages), float(diff_clip_ratio),
+                            float(pos_clip_ratio), float(neg_clip_ratio), float(final_clip_ratio), float(kl_coef),
+                            float(entropy_coef), float(grad_scale), _ptr(r.loss), _ptr(r.dloss), _ptr(r.kl),
+                            _ptr(r.is_positive_clipped), _ptr(r.is_negative_clipped), _ptr(r.is_clipped),
+                            _ptr(r.g_logprob), _ptr(r.g_entropy), _ptr(r.sums), _ptr(r.flags), _ptr(ws), ws.numel())
+    _lib.call("clgrpo_policy_loss", a, _stream(logprob))
+    return r
+
+
+# --------------------------------------------------------------------------- advantages
+
+def group_advantage(rewards, group_of, pool, pool_offsets, eps=1e-5):
+    """adv fp64 [n], all_zeros bool [n], all_ones bool [n]; all arguments device tensors."""
+    rewards = _dev(rewards, "rewards", torch.float64)
+    group_of = _dev(group_of, "group_of", torch.int32)
+    pool = _dev(pool, "pool", torch.float64)
+    pool_offsets = _dev(pool_offsets, "pool_offsets", torch.int32)
+    n = rewards.numel()
+    dev = rewards.device
+    adv = torch.empty(n, dtype=torch.float64, device=dev)
+    z = torch.empty(n, dtype=torch.bool, device=dev)
+    o = torch.empty(n, dtype=torch.bool, device=dev)
+    a = _lib.GroupAdvantageArgs(n, pool_offsets.numel() - 1, _ptr(rewards), _ptr(group_of), _ptr(pool),
+                                _ptr(pool_offsets), float(eps), _ptr(adv), _ptr(z), _ptr(o))
+    _lib.call("clgrpo_group_advantage", a, _stream(rewards))
+    return adv, z, o
+
+
+# --------------------------------------------------------------------------- masks / indices
+
+def build_masks(prompt_len: torch.Tensor, response_len: torch.Tensor, S: int, want_position_ids=True):
+    prompt_len = _dev(prompt_len, "prompt_len", torch.int32)
+    response_len = _dev(response_len, "response_len", torch.int32)
+    B = prompt_len.numel()
+    dev = prompt_len.device
+    attn = torch.empty(B, S, dtype=torch.int32, device=dev)
+    loss = torch.empty(B, S, dtype=torch.int32, device=dev)
+    pos = torch.empty(B, S, dtype=torch.int64, device=dev) if want_position_ids else None
+    a = _lib.BuildMasksArgs(B, S, _ptr(prompt_len), _ptr(response_len), _ptr(attn), _ptr(loss), _ptr(pos))
+    _lib.call("clgrpo_build_masks", a, _stream(prompt_len))
+    return attn, loss, pos
+
+
+def shift_labels(tokens: Optional[torch.Tensor], loss_mask: Optional[torch.Tensor], zero_last: bool):
+    ref = tokens if tokens is not None else loss_mask
+    B, S = ref.shape
+    labels = shifted = None
+    if tokens is not None:
+        tokens = _dev(tokens, "tokens", torch.int64)
+        labels = torch.empty_like(tokens)
+    if loss_mask is not None:
+        loss_mask = _dev(loss_mask, "loss_mask", torch.int32)
+        shifted = torch.empty_like(loss_mask)
+    a = _lib.ShiftLabelsArgs(B, S, _ptr(tokens), _ptr(loss_mask), _ptr(labels), _ptr(shifted), 1 if zero_last else 0)
+    _lib.call("clgrpo_shift_labels", a, _stream(ref))
+    return labels, shifted
+
+
+def unpad_indices(attn_mask: torch.Tensor):
+    """(indices int64 [T], cu_seqlens int32 [B+1], seqlens int32 [B], max_seqlen int) - one host sync."""
+    if attn_mask.dtype != torch.int32:
+        attn_mask = attn_mask.to(torch.int32)
+    attn_mask = _dev(attn_mask, "attention_mask", torch.int32)
+    B, S = attn_mask.shape
+    dev = attn_mask.device
+    indices = torch.empty(B * S, dtype=torch.int64, device=dev)
+    cu = torch.empty(B + 1, dtype=torch.int32, device=dev)
+    seqlens = torch.empty(B, dtype=torch.int32, device=dev)
+    total = torch.empty(2, dtype=torch.int32, device=dev)
+    row_off = torch.empty(B + 1, dtype=torch.int32, device=dev)
+    a = _lib.UnpadIndicesArgs(B, S, _ptr(attn_mask), _ptr(indices), _ptr(cu), _ptr(seqlens), _ptr(total), _ptr(row_off))
+    _lib.call("clgrpo_unpad_indices", a, _stream(attn_mask))
+    n_idx, max_len = total.tolist()
+    return indices[:n_idx], cu, seqlens, max_len
+
+
+def gather_rows(src: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    """src [N, ...] -> [len(indices), ...]"""
+    src = _dev(src, "src")
+    indices = _dev(indices, "indices", torch.int64)
+    row_shape = src.shape[1:]
+    row_bytes = src.element_size() * int(torch.Size(row_shape).numel())
+    out = torch.empty((indices.numel(),) + tuple(row_shape), dtype=src.dtype, device=src.device)
+    a = _lib.RowsArgs(_ptr(src), _ptr(out), _ptr(indices), indices.numel(), row_bytes, src.shape[0])
+    _lib.call("clgrpo_gather_rows", a, _stream(src))
+    return out
+
+
+def scatter_rows(src: torch.Tensor, indices: torch.Tensor, n_rows: int) -> torch.Tensor:
+    """zeros [n_rows, ...] with out[indices[i]] = src[i]"""
+    src = _dev(src, "src")
+    indices = _dev(indices, "indices", torch.int64)
+    row_shape = src.shape[1:]
+    row_bytes = src.element_size() * int(torch.Size(row_shape).numel())
+    out = torch.empty((n_rows,) + tuple(row_shape), dtype=src.dtype, device=src.device)
+    a = _lib.RowsArgs(_ptr(src), _ptr(out), _ptr(indices), indices.numel(), row_bytes, n_rows)
+    _lib.call("clgrpo_scatter_rows", a, _stream(src))
+    return out
+
+
+# --------------------------------------------------------------------------- host bin packing
+
+def _unflatten(order, offsets, n_bins) -> List[List[int]]:
+    return [list(order[offsets[b]:offsets[b + 1]]) for b in range(n_bins)]
+
+
+def bin_packing_ids(seq_len_list, max_train_token) -> List[List[int]]:
+    n = len(seq_len_list)
+    lens = (C.c_int64 * max(n, 1))(*[int(x) for x in seq_len_list])
+    order = (C.c_int64 * max(n, 1))()
+    offsets = (C.c_int64 * (n + 1))()
+    nb = C.c_int64(0)
+    _lib.check(_lib.lib().clgrpo_bin_packing(lens, n, int(max_train_token), order, offsets, C.byref(nb)))
+    return _unflatten(order, offsets, nb.value)
+
+
+def bin_packing_fix_bin_ids(seq_len_list, bin_size) -> List[List[int]]:
+    n = len(seq_len_list)
+    lens = (C.c_int64 * max(n, 1))(*[int(x) for x in seq_len_list])
+    order = (C.c_int64 * max(n, 1))()
+    offsets = (C.c_int64 * (int(bin_size) + 1))()
+    _lib.check(_lib.lib().clgrpo_bin_packing_fix_bin(lens, n, int(bin_size), order, offsets))
+    return _unflatten(order, offsets, int(bin_size))

@@ -1,0 +1,256 @@
+/* clgrpo.h - C ABI of the MI355X (gfx950) GRPO/GSPO policy-loss library.
+ *
+ * Plain C, no torch types.  Every tensor argument is a caller-owned pointer;
+ * device pointers unless the comment says "host".  Launching entry points take
+ * a hipStream_t (passed as void*) and only enqueue work on it.  They never
+ * allocate: scratch memory comes in through `workspace`, whose size the
+ * matching *_workspace_bytes() function reports.  Return value: 0, or a
+ * negative clgrpo_status; clgrpo_last_error_string() gives the reason for the
+ * calling thread.
+ *
+ * The reference (alibaba/ChatLearn) has no FFI: the functions named beside each
+ * entry point are the Python functions whose arithmetic the entry point
+ * replaces, paths relative to chatlearn/algorithm/grpo_utils/.
+ */
+#ifndef CLGRPO_H_
+#define CLGRPO_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  CLGRPO_OK = 0,
+  CLGRPO_EINVAL = -1,     /* bad scalar argument (negative size, bad mode, ...) */
+  CLGRPO_EDTYPE = -2,     /* unsupported dtype enum */
+  CLGRPO_ESHAPE = -3,     /* shape the kernels cannot take (e.g. H not a multiple of 64) */
+  CLGRPO_ENULL = -4,      /* required pointer is NULL */
+  CLGRPO_ELAUNCH = -5,    /* HIP reported an error at launch */
+  CLGRPO_EWORKSPACE = -6  /* workspace too small */
+} clgrpo_status;
+
+typedef enum { CLGRPO_BF16 = 0, CLGRPO_F32 = 1, CLGRPO_F64 = 2 } clgrpo_dtype;
+
+int clgrpo_version(void);
+const char* clgrpo_last_error_string(void);
+
+/* ------------------------------------------------------------------ *
+ * Fused lm_head projection + online log-softmax statistics.
+ * Replaces: model(...).logits (policy_trainer.py:216-221, nn.Linear(H,V)),
+ * logprobs_from_logits (trainer_utils.py:46-52), entropy_from_logits[_with_chunking]
+ * (trainer_utils.py:27-44), Megatron CE + _VocabParallelEntropy at tp=1
+ * (megatron_utils/train_helper.py:480-482,605-627).  The [T,V] logits are never
+ * written to memory.
+ * ------------------------------------------------------------------ */
+typedef struct {
+  const void* hidden;      /* [T, H] row-major, `dtype` */
+  const void* weight;      /* [V, H] row-major, `dtype` (lm_head.weight) */
+  const int64_t* labels;   /* [T]; NULL => logprob is not produced */
+  int64_t T, H, V;
+  int32_t dtype;           /* CLGRPO_BF16 or CLGRPO_F32 */
+  float inv_temperature;   /* logits are multiplied by this before the softmax (1/tau) */
+  float* logprob;          /* [T] out, fp32; may be NULL iff labels is NULL */
+  float* entropy;          /* [T] out, fp32; may be NULL */
+  float* rowmax;           /* [T] out, fp32 (max_v z); may be NULL */
+  float* lse;              /* [T] out, fp32 (logsumexp_v z); required */
+  void* workspace;
+  size_t workspace_bytes;
+} clgrpo_lmhead_fwd_args;
+
+size_t clgrpo_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype);
+int clgrpo_lmhead_fwd(const clgrpo_lmhead_fwd_args* a, void* stream);
+
+/* ------------------------------------------------------------------ *
+ * Backward of the fused head: recomputes logit tiles from hidden, W and the
+ * stored lse, forms d(logits) and contracts it into dhidden and dW.
+ * Replaces: autograd through lm_head / log_softmax / entropy at
+ * policy_trainer.py:286 (total_loss.backward()).
+ *   dz[t,v] = g_logprob[t] (1[v==label_t] - p[t,v]) - g_entropy[t] p[t,v] (log p[t,v] + entropy[t])
+ *   dhidden = inv_temperature * dz W        dW (+)= inv_temperature * dz^T hidden
+ * ------------------------------------------------------------------ */
+typedef struct {
+  const void* hidden;       /* [T, H] `dtype` */
+  const void* weight;       /* [V, H] `dtype` */
+  const int64_t* labels;    /* [T] */
+  const float* lse;         /* [T] from the forward */
+  const float* entropy;     /* [T] from the forward; required iff g_entropy != NULL */
+  const float* g_logprob;   /* [T] upstream gradient of logprob */
+  const float* g_entropy;   /* [T] upstream gradient of entropy, or NULL */
+  int64_t T, H, V;
+  int32_t dtype;
+  float inv_temperature;
+  void* dhidden;            /* [T, H] out, `dtype`; NULL => skipped */
+  float* dweight;           /* [V, H] out, fp32; NULL => skipped */
+  int32_t accumulate_dweight; /* nonzero: dweight += ; zero: dweight = */
+  void* workspace;
+  size_t workspace_bytes;   /* sets the token chunk: see clgrpo_lmhead_bwd_workspace_bytes */
+} clgrpo_lmhead_bwd_args;
+
+/* Bytes needed to process `chunk_tokens` tokens at a time (chunk_tokens <= 0: all T at once). */
+size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype,
+                                         int64_t chunk_tokens);
+int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream);
+
+/* ------------------------------------------------------------------ *
+ * Softmax statistics from materialised logits (legacy call sites that already
+ * hold [R, V] logits) and the matching backward.
+ * Replaces: logprobs_from_logits, entropy_from_logits, entropy_from_logits_with_chunking,
+ * entropy_from_tensor_parallel_logits (tp=1).
+ * ------------------------------------------------------------------ */
+typedef struct {
+  const void* logits;      /* [R, V] row-major with row stride `ld` elements */
+  const int64_t* labels;   /* [R] or NULL */
+  int64_t R, V, ld;
+  int32_t dtype;           /* CLGRPO_BF16 or CLGRPO_F32 */
+  float* logprob;          /* [R] or NULL */
+  float* entropy;          /* [R] or NULL */
+  float* lse;              /* [R] or NULL */
+} clgrpo_softmax_stats_args;
+int clgrpo_softmax_stats(const clgrpo_softmax_stats_args* a, void* stream);
+
+typedef struct {
+  const void* logits;      /* [R, V] */
+  const int64_t* labels;   /* [R] or NULL (required iff g_logprob) */
+  const float* g_logprob;  /* [R] or NULL */
+  const float* g_entropy;  /* [R] or NULL */
+  int64_t R, V, ld;
+  int32_t dtype;
+  void* dlogits;           /* [R, V] out, `dtype`, row stride V */
+} clgrpo_softmax_stats_bwd_args;
+int clgrpo_softmax_stats_bwd(const clgrpo_softmax_stats_bwd_args* a, void* stream);
+
+/* ------------------------------------------------------------------ *
+ * Clipped importance-ratio policy loss (token-level GRPO or sequence-level
+ * GSPO), k3 KL estimator, masked sums and the per-token upstream gradients.
+ * Replaces: calculate_grpo_loss (loss_gallery.py:6-33), calculate_gspo_loss
+ * (loss_gallery.py:35-74), the loss assembly of policy_trainer.py:263-286 and
+ * _compute_all_losses / loss_func of megatron_utils/train_helper.py:426-547.
+ *
+ * Tokens are addressed flat, n = total elements.  Sequence of token i:
+ *   cu_seqlens != NULL : packed, the b with cu_seqlens[b] <= i < cu_seqlens[b+1]
+ *   cu_seqlens == NULL : padded [B, S] row-major, b = i / S.
+ * ------------------------------------------------------------------ */
+typedef enum { CLGRPO_LOSS_GRPO = 0, CLGRPO_LOSS_GSPO = 1 } clgrpo_loss_mode;
+
+typedef struct {
+  int32_t mode;              /* clgrpo_loss_mode */
+  int32_t compute_dtype;     /* CLGRPO_F32 or CLGRPO_F64: type of advantages, loss, dloss */
+  int64_t n;                 /* tokens */
+  int64_t B;                 /* sequences */
+  int64_t S;                 /* padded row length (used iff cu_seqlens == NULL) */
+  const int32_t* cu_seqlens; /* [B+1] or NULL */
+  const float* logprob;      /* [n] */
+  const float* old_logprob;  /* [n] */
+  const float* ref_logprob;  /* [n] or NULL (no KL term) */
+  const float* entropy;      /* [n] or NULL */
+  const int32_t* loss_mask;  /* [n] or NULL (= all ones) */
+  const void* advantages;    /* [B] compute_dtype */
+  double diff_clip_ratio, pos_clip_ratio, neg_clip_ratio, final_clip_ratio;
+  double kl_coef, entropy_coef; /* used only for g_logprob / g_entropy */
+  double grad_scale;         /* fsdp_size / N of policy_trainer.py:266-285 */
+  void* loss;                /* [n] out compute_dtype: per-token surrogate (unmasked) */
+  void* dloss_dlogprob;      /* [n] out compute_dtype or NULL: d loss[i] / d logprob[i] */
+  float* kl;                 /* [n] out fp32 or NULL: clamp(exp(k)-k-1,-10,10), k=ref-lp,
+                                with exp(k) replaced by 1 where the mask is 0 (train_helper.py:524) */
+  uint8_t* is_positive_clipped; /* [n] or NULL (GSPO flags; also defined for GRPO) */
+  uint8_t* is_negative_clipped; /* [n] or NULL */
+  uint8_t* is_clipped;          /* [n] or NULL */
+  float* g_logprob;          /* [n] out or NULL: mask*grad_scale*(dloss + kl_coef*dkl) */
+  float* g_entropy;          /* [n] out or NULL: -entropy_coef*mask*grad_scale */
+  double* sums;              /* [8] out: sum(mask*loss), sum(mask*kl), sum(mask*entropy), sum(mask),
+                                sum(mask*pos), sum(mask*neg), sum(mask*clipped), 0 */
+  int32_t* flags;            /* [1] out: bit0 loss has NaN, bit1 exp(k) has Inf, bit2 exp(k) has NaN */
+  void* workspace;
+  size_t workspace_bytes;
+} clgrpo_policy_loss_args;
+
+size_t clgrpo_policy_loss_workspace_bytes(int64_t n, int64_t B);
+int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream);
+
+/* ------------------------------------------------------------------ *
+ * Group-wise reward -> advantage: adv = (r - mean(pool_g)) / (std(pool_g) + eps),
+ * population std, float64.  Replaces: AdvantageComputer.__call__ arithmetic
+ * (advantage_compute.py:27-36).  pool holds, group after group, every reward
+ * buffered for that prompt (this call's and carried-over ones).
+ * ------------------------------------------------------------------ */
+typedef struct {
+  int64_t n_samples, n_groups;
+  const double* rewards;      /* [n_samples] */
+  const int32_t* group_of;    /* [n_samples] group index of each sample */
+  const double* pool;         /* [pool_offsets[n_groups]] */
+  const int32_t* pool_offsets;/* [n_groups+1] */
+  double eps;
+  double* advantages;         /* [n_samples] out */
+  uint8_t* all_zeros;         /* [n_samples] out: every pooled reward of the group == 0 */
+  uint8_t* all_ones;          /* [n_samples] out: every pooled reward of the group == 1 */
+} clgrpo_group_advantage_args;
+int clgrpo_group_advantage(const clgrpo_group_advantage_args* a, void* stream);
+
+/* ------------------------------------------------------------------ *
+ * Mask / index builders for padded <-> packed batches (bit-exact integers).
+ * Replaces: generate_loss_mask_position_ids (trainer_utils.py:60-96, text branch),
+ * the label roll and training-mask shift (policy_trainer.py:135,160-162;
+ * train_helper.py:405-413), unpad_input (trainer_utils.py:155-194) and the
+ * flash-attn index_first_axis / pad_input it relies on.
+ * ------------------------------------------------------------------ */
+typedef struct {
+  int64_t B, S;
+  const int32_t* prompt_len;   /* [B] */
+  const int32_t* response_len; /* [B] */
+  int32_t* attn_mask;          /* [B,S] out */
+  int32_t* loss_mask;          /* [B,S] out */
+  int64_t* position_ids;       /* [B,S] out or NULL */
+} clgrpo_build_masks_args;
+int clgrpo_build_masks(const clgrpo_build_masks_args* a, void* stream);
+
+typedef struct {
+  int64_t B, S;
+  const int64_t* tokens;       /* [B,S] or NULL */
+  const int32_t* loss_mask;    /* [B,S] or NULL */
+  int64_t* labels;             /* [B,S] out: tokens rolled left by one along S (wraps) */
+  int32_t* shifted_mask;       /* [B,S] out: mask rolled left by one along S */
+  int32_t zero_last;           /* nonzero: shifted_mask[:, S-1] = 0 (FSDP trainer) */
+} clgrpo_shift_labels_args;
+int clgrpo_shift_labels(const clgrpo_shift_labels_args* a, void* stream);
+
+typedef struct {
+  int64_t B, S;
+  const int32_t* attn_mask;    /* [B,S] */
+  int64_t* indices;            /* [B*S] out: flat positions of the nonzero mask entries, ascending;
+                                  only the first total[0] are written */
+  int32_t* cu_seqlens;         /* [B+1] out */
+  int32_t* seqlens;            /* [B] out */
+  int32_t* total;              /* [2] out: {number of indices written, max seqlen} */
+  int32_t* row_offsets;        /* [B+1] scratch */
+} clgrpo_unpad_indices_args;
+int clgrpo_unpad_indices(const clgrpo_unpad_indices_args* a, void* stream);
+
+typedef struct {
+  const void* src;             /* gather: [n_src_rows, row_bytes]; scatter: [n_idx, row_bytes] */
+  void* dst;                   /* gather: [n_idx, row_bytes];      scatter: [n_dst_rows, row_bytes] */
+  const int64_t* indices;      /* [n_idx] */
+  int64_t n_idx, row_bytes;
+  int64_t n_rows;              /* rows of the indexed side (bounds check on the host is the caller's) */
+} clgrpo_rows_args;
+int clgrpo_gather_rows(const clgrpo_rows_args* a, void* stream);   /* dst[i] = src[indices[i]] */
+int clgrpo_scatter_rows(const clgrpo_rows_args* a, void* stream);  /* dst = 0; dst[indices[i]] = src[i] */
+
+/* ------------------------------------------------------------------ *
+ * Host-side bin packing for dynamic batching (runs on the CPU, like the
+ * reference's).  Replaces: bin_packing (packing_utils.py:23-54) and
+ * bin_packing_fix_bin (packing_utils.py:56-83).  All pointers are HOST memory.
+ * bin_of[i] receives the bin of item i; order[] receives the item ids bin after
+ * bin in insertion order, bin_offsets[b]..bin_offsets[b+1] delimiting bin b.
+ * ------------------------------------------------------------------ */
+int clgrpo_bin_packing(const int64_t* seq_len, int64_t n, int64_t max_train_token,
+                       int64_t* order, int64_t* bin_offsets, int64_t* n_bins);
+int clgrpo_bin_packing_fix_bin(const int64_t* seq_len, int64_t n, int64_t bin_size,
+                               int64_t* order, int64_t* bin_offsets);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CLGRPO_H_ */

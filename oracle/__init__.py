@@ -1,0 +1,26 @@
+"""CPU oracle for the GRPO/GSPO policy-loss path.  TEST INFRASTRUCTURE ONLY.
+
+This package restates, with torch/numpy on the CPU, what the reference's
+``chatlearn/algorithm/grpo_utils`` functions compute.  It exists so that the
+HIP kernels can be checked against it; nothing under ``chatlearn_amd/`` may
+import it.  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` use it, and there only as the checker or
+as the timed CPU baseline.
+
+How each function is pinned (the reference's own tests hold no vector for any
+of them, so none is pinned by a reference fixture):
+
+* softmax statistics (logprob, entropy) and their gradients: closed forms
+  (uniform logits, one dominant logit, shift invariance, zero-sum gradient),
+  a pure-Python row loop on tiny shapes, and torch's library routines.
+* GRPO / GSPO surrogate losses: closed forms for every clip branch
+  (``tests/test_oracle_losses.py``) and torch autograd for the tie gradients.
+* k3 KL estimator: ``kl >= 0``, zero iff equal, derivative ``1 - exp(ref-lp)``.
+* bin packing: hand-worked cases stored in ``tests/golden/packing_cases.json``
+  that exercise the strict-fit rule, first-on-ties and stable descending
+  order, plus invariants on random inputs.
+* masks / unpad / pad: brute-force nested loops on tiny shapes and the
+  round-trip ``pad(unpad(x)) == x * mask``.
+* group advantages: ``numpy.mean`` / ``numpy.std`` and the Bernoulli closed
+  form ``(1-k/G)/(sqrt(k/G(1-k/G))+1e-5)``.
+"""

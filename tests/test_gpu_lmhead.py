@@ -1,0 +1,136 @@
+"""Fused lm_head forward / backward (HIP, through the C ABI) against the CPU oracle
+on identical seeded inputs.  Tolerances: 1e-5 relative in fp32, 1e-2 relative in
+bf16 (relative to the largest magnitude of the compared tensor)."""
+import math
+
+import pytest
+import torch
+
+from oracle import softmax_stats as osm
+from tests.util import assert_close_rel
+
+pytestmark = pytest.mark.gpu
+
+RTOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2}
+
+
+def _inputs(T, H, V, dtype, seed, w_std=0.05):
+    g = torch.Generator().manual_seed(seed)
+    hidden = torch.randn(T, H, generator=g).to(dtype)
+    weight = (torch.randn(V, H, generator=g) * w_std).to(dtype)
+    labels = torch.randint(0, V, (T,), generator=g)
+    # make sure the edges of the vocabulary are hit
+    labels[0], labels[-1] = 0, V - 1
+    return hidden, weight, labels
+
+
+CASES = [
+    # T, H, V, dtype, temperature
+    (300, 256, 5000, torch.float32, 1.0),      # ragged T and V
+    (1, 64, 257, torch.float32, 1.0),          # single token, V just past one tile
+    (513, 128, 1000, torch.float32, 0.7),      # temperature
+    (300, 256, 5000, torch.bfloat16, 1.0),
+    (700, 512, 9001, torch.bfloat16, 0.7),
+    (256, 1024, 4096, torch.bfloat16, 1.0),    # exact tiles
+]
+
+
+@pytest.mark.parametrize("T,H,V,dtype,temp", CASES)
+def test_forward_matches_oracle(dev, T, H, V, dtype, temp):
+    from chatlearn_amd import ops
+    hidden, weight, labels = _inputs(T, H, V, dtype, seed=T + V)
+    lp, ent, mx, lse = ops.lmhead_forward(hidden.to(dev), weight.to(dev), labels.to(dev), temp, need_entropy=True)
+    rlp, rent, rmx, rlse = osm.fused_head_forward(hidden, weight, labels, temp, torch.float64)
+    r = RTOL[dtype]
+    assert_close_rel(lp, rlp, r, "logprob")
+    assert_close_rel(ent, rent, r, "entropy")
+    assert_close_rel(lse, rlse, r, "lse")
+    assert_close_rel(mx, rmx, r, "rowmax")
+    assert (lp <= 1e-6).all() and (ent >= -1e-6).all() and (ent <= math.log(V) + 1e-4).all()
+
+
+@pytest.mark.parametrize("T,H,V,dtype,temp", CASES)
+@pytest.mark.parametrize("with_entropy", [False, True])
+def test_backward_matches_oracle(dev, T, H, V, dtype, temp, with_entropy):
+    from chatlearn_amd import ops
+    hidden, weight, labels = _inputs(T, H, V, dtype, seed=T + V + 1)
+    g = torch.Generator().manual_seed(5)
+    g_lp = torch.randn(T, generator=g)
+    g_lp[torch.rand(T, generator=g) < 0.3] = 0.0          # masked-out tokens
+    g_ent = torch.randn(T, generator=g) * 0.1 if with_entropy else None
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld, temp, need_entropy=True)
+    dh, dw = ops.lmhead_backward(hd, wd, ld, lse, ent, g_lp.to(dev), g_ent.to(dev) if with_entropy else None, temp)
+    rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, g_lp, g_ent, temp)
+    r = RTOL[dtype]
+    assert dh.dtype == dtype and dw.dtype == torch.float32
+    assert_close_rel(dh, rdh, r, "dhidden")
+    assert_close_rel(dw, rdw, r, "dweight")
+
+
+def test_backward_chunked_equals_unchunked_and_accumulates(dev):
+    from chatlearn_amd import ops
+    T, H, V = 900, 256, 3000
+    hidden, weight, labels = _inputs(T, H, V, torch.bfloat16, seed=3)
+    g_lp = torch.randn(T, generator=torch.Generator().manual_seed(1))
+    hd, wd, ld, gd = hidden.to(dev), weight.to(dev), labels.to(dev), g_lp.to(dev)
+    lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld)
+    dh1, dw1 = ops.lmhead_backward(hd, wd, ld, lse, None, gd)
+    dh2, dw2 = ops.lmhead_backward(hd, wd, ld, lse, None, gd, chunk_tokens=256)
+    assert torch.equal(dh1, dh2)                      # dhidden rows do not depend on the chunking
+    assert_close_rel(dw2, dw1, 1e-5, "chunked dW")   # only the fp32 summation order differs
+    base = torch.ones(V, H, device=dev)
+    _, dw3 = ops.lmhead_backward(hd, wd, ld, lse, None, gd, dweight=base, accumulate_dweight=True)
+    assert dw3.data_ptr() == base.data_ptr()
+    assert_close_rel(dw3 - 1.0, dw1, 1e-4, "accumulated dW")
+
+
+def test_closed_forms(dev):
+    """Uniform logits: lp = -log V, entropy = log V.  One dominant logit: lp -> 0, entropy -> 0."""
+    from chatlearn_amd import ops
+    T, H, V = 64, 64, 777
+    hidden = torch.zeros(T, H, device=dev)
+    weight = torch.randn(V, H, device=dev)
+    labels = torch.randint(0, V, (T,), device=dev)
+    lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels)
+    assert torch.allclose(lp, torch.full_like(lp, -math.log(V)), atol=1e-5)
+    assert torch.allclose(ent, torch.full_like(ent, math.log(V)), atol=1e-5)
+    hidden = torch.zeros(T, H, device=dev)
+    hidden[:, 0] = 1.0
+    weight = torch.zeros(V, H, device=dev)
+    weight[5, 0] = 60.0
+    labels = torch.full((T,), 5, device=dev)
+    lp, ent, _, _ = ops.lmhead_forward(hidden, weight, labels)
+    assert lp.abs().max() < 1e-5 and ent.abs().max() < 1e-5
+
+
+def test_autograd_function_matches_oracle_autograd(dev):
+    from chatlearn_amd import fused_linear_logprob_entropy
+    T, H, V = 260, 128, 1500
+    hidden, weight, labels = _inputs(T, H, V, torch.float32, seed=11)
+    h = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    lp, ent = fused_linear_logprob_entropy(h.view(2, 130, H), w, labels.to(dev).view(2, 130), temperature=0.9)
+    assert lp.shape == (2, 130) and ent.shape == (2, 130)
+    g = torch.Generator().manual_seed(2)
+    c_lp, c_ent = torch.randn(T, generator=g), torch.randn(T, generator=g)
+    ((lp.reshape(-1) * c_lp.to(dev)).sum() + (ent.reshape(-1) * c_ent.to(dev)).sum()).backward()
+    rdh, rdw = osm.fused_head_backward_autograd(hidden, weight, labels, c_lp, c_ent, 0.9)
+    assert_close_rel(h.grad, rdh, 1e-5, "hidden.grad")
+    assert_close_rel(w.grad, rdw, 1e-5, "weight.grad")
+
+
+def test_argument_errors(dev):
+    from chatlearn_amd import ops
+    from chatlearn_amd._lib import ClgrpoError
+    h = torch.zeros(4, 48, device=dev)
+    w = torch.zeros(10, 48, device=dev)
+    with pytest.raises(ClgrpoError, match="ESHAPE"):
+        ops.lmhead_forward(h, w, torch.zeros(4, dtype=torch.int64, device=dev))
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.lmhead_forward(torch.zeros(4, 64), torch.zeros(10, 64), None)
+    # a label outside the vocabulary is flagged with NaN instead of a silent number
+    h = torch.randn(4, 64, device=dev)
+    w = torch.randn(10, 64, device=dev)
+    lp, *_ = ops.lmhead_forward(h, w, torch.tensor([0, 9, 10, -1], device=dev))
+    assert torch.isfinite(lp[:2]).all() and torch.isnan(lp[2:]).all()
