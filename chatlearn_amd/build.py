@@ -29,6 +29,8 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON_FLAGS = ["-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function"]
 # Packed-fp32 instruction selection is switched off for all device code.
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# advantage.hip reproduces numpy's float64 rounding step by step: no fused multiply-adds there.
+PER_FILE_FLAGS = {"advantage.hip": ["-ffp-contract=off"]}
 
 
 def _compile(src):
@@ -36,6 +38,7 @@ def _compile(src):
     cmd = [HIPCC] + COMMON_FLAGS
     if src.endswith(".hip"):
         cmd += DEVICE_FLAGS
+    cmd += PER_FILE_FLAGS.get(src, [])
     cmd += ["-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"

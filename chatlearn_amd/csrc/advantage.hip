@@ -3,8 +3,8 @@
 // One thread per sample walks the pooled rewards of the sample's group (a group
 // is the 8-32 responses of one prompt, so the pool sits in L2).  Sums follow
 // numpy's pairwise scheme for blocks of up to 128 values (eight running sums,
-// then a fixed tree), with explicitly rounded adds/multiplies so the compiler
-// cannot contract them into FMAs; the result is numpy.mean / numpy.std bit for
+// then a fixed tree), and this file is compiled with -ffp-contract=off so no add is fused with
+// a multiply; the result is numpy.mean / numpy.std bit for
 // bit for pools of at most 128 rewards and differs only by summation order above.
 #include "common.hpp"
 

@@ -17,7 +17,6 @@ namespace clgrpo {
 
 constexpr int kFwdBM = 256, kFwdBN = 256;
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
 
 struct FwdParams {
   const void* hidden;
