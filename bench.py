@@ -149,6 +149,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-unfused", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256)
+    ap.add_argument("--no-skip-masked", action="store_true",
+                    help="run the backward on every row, also those whose loss mask is zero")
+    ap.add_argument("--keep-logits-chunk", type=int, default=8192,
+                    help="tokens per chunk whose logits the forward keeps for the backward (0: recompute)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives are built); use --gpus 1", file=sys.stderr)
@@ -167,50 +171,68 @@ def main():
     lp0, *_ = ops.lmhead_forward(hidden, weight, labels, cfg.temperature, need_entropy=False)
     old, ref = synthetic.noisy_logprobs(lp0, synthetic.generator_for(cfg))
     dweight = torch.zeros(cfg.V, cfg.H, dtype=torch.float32, device=dev) if train else None
-    mode = LOSS_GSPO if cfg.loss == "gspo" else LOSS_GRPO
 
-    stage_events = []
+    from chatlearn_amd.fused import grpo_head_step, _token_chunks
+    keep = args.keep_logits_chunk if (train and args.keep_logits_chunk > 0) else None
+    cu_host = cu.tolist()
+    chunks = _token_chunks(T, keep, cu_host if (keep and cfg.loss == "gspo") else None)
+    marks = []
 
     def step(record=False):
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if record else None
-        if record:
-            ev[0].record()
-        lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, cfg.temperature, need_entropy=True)
-        if record:
-            ev[1].record()
-        if train:
-            res = ops.policy_loss(lp, old, adv, mode=mode, cu_seqlens=cu, ref_logprob=ref, entropy=ent,
-                                  loss_mask=mask, diff_clip_ratio=cfg.diff_clip_ratio,
-                                  pos_clip_ratio=cfg.pos_clip_ratio, neg_clip_ratio=cfg.neg_clip_ratio,
-                                  final_clip_ratio=cfg.final_clip_ratio, kl_coef=cfg.kl_coef,
-                                  entropy_coef=cfg.entropy_coef, grad_scale=1.0 / n_tok, want_dloss=False,
-                                  want_upstream=True)
+        """One pass of the head over the micro-batch.  Training configurations: per token chunk,
+        fused forward (keeping the chunk's logits), loss + upstream gradients, fused backward
+        (dhidden, dW accumulated).  The no-grad configuration: fused forward only."""
+        if not train:
             if record:
-                ev[2].record()
-            ops.lmhead_backward(hidden, weight, labels, lse, ent, res.g_logprob, res.g_entropy, cfg.temperature,
-                                need_dhidden=True, need_dweight=True, dweight=dweight, accumulate_dweight=False)
-        elif record:
-            ev[2].record()
-        if record:
-            ev[3].record()
-            stage_events.append(ev)
+                e = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+                e[0].record()
+            ops.lmhead_forward(hidden, weight, labels, cfg.temperature, need_entropy=True)
+            if record:
+                e[1].record()
+                marks.append([("forward", e[0]), ("end", e[1])])
+            return None
+        cur = []
 
+        def hook(name):
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            cur.append((name, ev))
+        out = grpo_head_step(hidden, weight, labels, old, ref, adv, cu, mask, n_tokens_total=n_tok,
+                             use_group_sequence_policy=(cfg.loss == "gspo"), pos_clip_ratio=cfg.pos_clip_ratio,
+                             neg_clip_ratio=cfg.neg_clip_ratio, diff_clip_ratio=cfg.diff_clip_ratio,
+                             final_clip_ratio=cfg.final_clip_ratio, kl_coef=cfg.kl_coef,
+                             entropy_coef=cfg.entropy_coef, temperature=cfg.temperature, dweight=dweight,
+                             accumulate_dweight=False, keep_logits_chunk=keep, cu_seqlens_host=cu_host,
+                             skip_masked_rows=not args.no_skip_masked, stage_hook=hook if record else None,
+                             check_flags=False)
+        if record:
+            marks.append(cur)
+        return out
+
+    out_last = None
     for _ in range(args.warmup):
-        step()
+        out_last = step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step(record=True)
+        out_last = step(record=True)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
 
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in stage_events) / len(stage_events)
-    loss_ms = sum(e[1].elapsed_time(e[2]) for e in stage_events) / len(stage_events)
-    bwd_ms = sum(e[2].elapsed_time(e[3]) for e in stage_events) / len(stage_events)
+    def stage_ms(name):
+        tot = 0.0
+        for cur in marks:
+            for (a, ea), (_, eb) in zip(cur[:-1], cur[1:]):
+                if a == name:
+                    tot += ea.elapsed_time(eb)
+        return tot / len(marks)
+    fwd_ms, loss_ms, bwd_ms = stage_ms("forward"), stage_ms("loss"), stage_ms("backward")
+    n_fwd_launch = len(chunks) if train else 1
+    rows_bwd = out_last["rows_projected_bwd"] if train else 0
 
     thv = float(T) * cfg.H * cfg.V
     peak = PEAK_BF16_TFLOPS if cfg.dtype == torch.bfloat16 else PEAK_F32_TFLOPS
-    fwd_tflops = 2.0 * thv / (fwd_ms * 1e-3) / 1e12
+    fwd_tflops = 2.0 * thv / (fwd_ms * 1e-3) / 1e12          # all forward launches of a step together
     step_flops = (6.0 if train else 2.0) * thv
     out = {
         "metric": "packed tokens/sec, fused logprob+GRPO loss fwd+bwd (Qwen3-8B head); % MFMA peak",
@@ -228,10 +250,13 @@ def main():
         "config": {"workload": f"{cfg.name}: H={cfg.H} V={cfg.V} T={T} packed tokens in {len(samples)} sequences, "
                                f"{cfg.loss or 'no-grad logprob+entropy'}"
                                f"{' fwd+bwd (dhidden ' + str(cfg.dtype).split('.')[-1] + ', dW fp32)' if train else ''}",
-                   "temperature": cfg.temperature, "kl_coef": cfg.kl_coef, "entropy_coef": cfg.entropy_coef},
+                   "temperature": cfg.temperature, "kl_coef": cfg.kl_coef, "entropy_coef": cfg.entropy_coef,
+                   "token_chunks": [hi - lo for lo, hi in chunks], "logits_kept_per_chunk": bool(keep),
+                   "T_projected_forward": T, "T_projected_backward": rows_bwd},
         "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tflops, "peak": peak,
                      "unit": "TFLOP/s", "frac": fwd_tflops / peak, "traffic": None,
-                     "algorithmic_flops_per_launch": 2.0 * thv, "avg_launch_ms": fwd_ms},
+                     "algorithmic_flops_per_launch": 2.0 * thv / n_fwd_launch,
+                     "avg_launch_ms": fwd_ms / n_fwd_launch, "launches_per_step": n_fwd_launch},
         "step_mfma_frac": step_flops / dt / 1e12 / peak,
         "stage_ms": {"forward": fwd_ms, "loss": loss_ms, "backward": bwd_ms},
     }

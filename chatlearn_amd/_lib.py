@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libclgrpo.so")
+# CLGRPO_LIB_PATH selects another build of the same library (e.g. a tuning variant).
+LIB_PATH = os.environ.get("CLGRPO_LIB_PATH") or os.path.join(_HERE, "csrc", "libclgrpo.so")
 
 BF16, F32, F64 = 0, 1, 2
 LOSS_GRPO, LOSS_GSPO = 0, 1
@@ -28,14 +29,16 @@ class ClgrpoError(RuntimeError):
 class LmheadFwdArgs(C.Structure):
     _fields_ = [("hidden", vp), ("weight", vp), ("labels", vp), ("T", i64), ("H", i64), ("V", i64),
                 ("dtype", i32), ("inv_temperature", f32), ("logprob", vp), ("entropy", vp),
-                ("rowmax", vp), ("lse", vp), ("workspace", vp), ("workspace_bytes", sz)]
+                ("rowmax", vp), ("lse", vp), ("workspace", vp), ("workspace_bytes", sz),
+                ("saved_logits", vp), ("ld_saved", i64), ("saved_row_map", vp), ("saved_rows", i64)]
 
 
 class LmheadBwdArgs(C.Structure):
     _fields_ = [("hidden", vp), ("weight", vp), ("labels", vp), ("lse", vp), ("entropy", vp),
                 ("g_logprob", vp), ("g_entropy", vp), ("T", i64), ("H", i64), ("V", i64),
                 ("dtype", i32), ("inv_temperature", f32), ("dhidden", vp), ("dweight", vp),
-                ("accumulate_dweight", i32), ("workspace", vp), ("workspace_bytes", sz)]
+                ("accumulate_dweight", i32), ("workspace", vp), ("workspace_bytes", sz),
+                ("saved_logits", vp), ("ld_saved", i64), ("weight_t", vp), ("weight_t_ready", i32)]
 
 
 class SoftmaxStatsArgs(C.Structure):
@@ -56,7 +59,8 @@ class PolicyLossArgs(C.Structure):
                 ("final_clip_ratio", f64), ("kl_coef", f64), ("entropy_coef", f64), ("grad_scale", f64),
                 ("loss", vp), ("dloss_dlogprob", vp), ("kl", vp), ("is_positive_clipped", vp),
                 ("is_negative_clipped", vp), ("is_clipped", vp), ("g_logprob", vp), ("g_entropy", vp),
-                ("sums", vp), ("flags", vp), ("workspace", vp), ("workspace_bytes", sz)]
+                ("sums", vp), ("flags", vp), ("workspace", vp), ("workspace_bytes", sz),
+                ("token_offset", i64)]
 
 
 class GroupAdvantageArgs(C.Structure):
@@ -89,7 +93,8 @@ SIGNATURES = {
     "clgrpo_last_error_string": (C.c_char_p, []),
     "clgrpo_lmhead_fwd_workspace_bytes": (sz, [i64, i64, i64, i32]),
     "clgrpo_lmhead_fwd": (C.c_int, [C.POINTER(LmheadFwdArgs), vp]),
-    "clgrpo_lmhead_bwd_workspace_bytes": (sz, [i64, i64, i64, i32, i64]),
+    "clgrpo_saved_logits_ld": (i64, [i64]),
+    "clgrpo_lmhead_bwd_workspace_bytes": (sz, [i64, i64, i64, i32, i64, i32]),
     "clgrpo_lmhead_bwd": (C.c_int, [C.POINTER(LmheadBwdArgs), vp]),
     "clgrpo_softmax_stats": (C.c_int, [C.POINTER(SoftmaxStatsArgs), vp]),
     "clgrpo_softmax_stats_bwd": (C.c_int, [C.POINTER(SoftmaxStatsBwdArgs), vp]),

@@ -52,8 +52,8 @@ struct DzParams {
 };
 
 template <typename T>
-__global__ __launch_bounds__(512) void lmhead_dz_kernel(DzParams p) {
-  using Tile = GemmTile<T, 256, 256, 2, 4>;
+__global__ __launch_bounds__(kHeadThreads) void lmhead_dz_kernel(DzParams p) {
+  using Tile = HeadTile<T>;
   constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
   extern __shared__ __align__(16) char lds[];
 
@@ -138,6 +138,74 @@ __global__ __launch_bounds__(512) void lmhead_dz_kernel(DzParams p) {
   }
 }
 
+// d(logits) from stored logits, in place, plus its transpose.  One 64 x 64 (token x vocabulary)
+// tile per workgroup: read z (16 bytes per lane along the vocabulary), form dz with the per-token
+// coefficients, write it back over z, and turn the tile through LDS so dzT[vocab][token] is also
+// written in 16-byte pieces.  HBM-bound: reads 1x, writes 2x the chunk.
+struct DzFromZParams {
+  void* z;            // [Tc][ldv] in: raw logits, out: dz
+  void* dzT;          // [V][ldt]
+  const int64_t* labels;
+  const float* lse;
+  const float* entropy;
+  const float* g_lp;
+  const float* g_ent;
+  int Tc, ldt, V, ldv;
+  float c, inv_temperature;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void dz_from_z_kernel(DzFromZParams p) {
+  constexpr int VEC = 16 / (int)sizeof(T);       // elements per 16-byte access
+  constexpr int CPR = 64 / VEC;                  // accesses per 64-wide tile row
+  constexpr int RPP = 256 / CPR;                 // tile rows covered per pass
+  __shared__ T tile[64][64 + VEC];               // [vocab][token], padded rows
+  const int t0 = blockIdx.x * 64, v0 = blockIdx.y * 64;
+  const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
+  T* z = static_cast<T*>(p.z);
+  T* dzT = static_cast<T*>(p.dzT);
+  const float it = p.inv_temperature;
+  for (int rr = r; rr < 64; rr += RPP) {
+    const int t = t0 + rr;
+    const int v = v0 + c * VEC;
+    alignas(16) T vals[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) vals[j] = (T)0.f;
+    if (t < p.Tc && v < p.ldv) {
+      const float glp = p.g_lp[t];
+      const float gen = p.g_ent ? p.g_ent[t] : 0.f;
+      if (glp != 0.f || gen != 0.f) {
+        const float lse = p.lse[t];
+        const float lse2 = lse * kLog2e;
+        const float ent = p.g_ent ? p.entropy[t] : 0.f;
+        const int64_t lab = p.labels[t];
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(z + (int64_t)t * p.ldv + v);
+        const T* in = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float zraw = (float)in[j];
+          const float pr = __builtin_amdgcn_exp2f(fmaf(zraw, p.c, -lse2));
+          const float logp = fmaf(zraw, it, -lse);
+          float d = -it * pr * fmaf(gen, logp + ent, glp);
+          if (v + j == lab) d += it * glp;
+          if (v + j >= p.V) d = 0.f;
+          vals[j] = (T)d;
+        }
+      }
+      *reinterpret_cast<u32x4*>(z + (int64_t)t * p.ldv + v) = *reinterpret_cast<const u32x4*>(vals);
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) tile[c * VEC + j][rr] = vals[j];
+  }
+  __syncthreads();
+  for (int rr = r; rr < 64; rr += RPP) {
+    const int v = v0 + rr;
+    const int t = t0 + c * VEC;
+    if (v < p.V && t < p.ldt)
+      *reinterpret_cast<u32x4*>(dzT + (int64_t)v * p.ldt + t) = *reinterpret_cast<const u32x4*>(&tile[rr][c * VEC]);
+  }
+}
+
 // C[m][n] (+)= alpha * sum_k A[m][k] B[n][k];  C row-major with leading dimension ldc.
 struct GemmParams {
   const void* A;
@@ -147,6 +215,9 @@ struct GemmParams {
   int M, N, K;
   int n_mt, n_nt;
   int accumulate;
+  int k_split;        // > 1: work item = (tile, K range); fp32 partial tiles go to `partial`
+  int k_per_split;    // K extent of one range, a multiple of the slab
+  float* partial;     // [k_split][M][N] fp32, row stride N
 };
 
 template <typename OutT> __device__ __forceinline__ OutT cvt_out(float v);
@@ -154,13 +225,15 @@ template <> __device__ __forceinline__ float cvt_out<float>(float v) { return v;
 template <> __device__ __forceinline__ __bf16 cvt_out<__bf16>(float v) { return (__bf16)v; }
 
 template <typename T, typename OutT>
-__global__ __launch_bounds__(512) void gemm_nt_kernel(GemmParams p) {
-  using Tile = GemmTile<T, 256, 256, 2, 4>;
+__global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
+  using Tile = HeadTile<T>;
   constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
   extern __shared__ __align__(16) char lds[];
 
-  const int item = xcd_remap(blockIdx.x, gridDim.x);
-  if (item >= p.n_mt * p.n_nt) return;
+  int item = xcd_remap(blockIdx.x, gridDim.x);
+  if (item >= p.n_mt * p.n_nt * p.k_split) return;
+  const int ks = item / (p.n_mt * p.n_nt);
+  item -= ks * (p.n_mt * p.n_nt);
   int mt, nt;
   grouped_tile(item, p.n_mt, p.n_nt, 8, mt, nt);
   const int lane = threadIdx.x & 63;
@@ -169,6 +242,8 @@ __global__ __launch_bounds__(512) void gemm_nt_kernel(GemmParams p) {
   const int m0 = mt * 256, n0 = nt * 256;
   const int a_rows = (p.M - m0) < 256 ? (p.M - m0) : 256;
   const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
+  const int k0 = ks * p.k_per_split;
+  const int k_len = (p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split;
 
   f32x16 acc[MI][NI];
 #pragma unroll
@@ -178,8 +253,25 @@ __global__ __launch_bounds__(512) void gemm_nt_kernel(GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
-  Tile::run(acc, static_cast<const T*>(p.A) + (int64_t)m0 * p.lda, p.lda, a_rows,
-            static_cast<const T*>(p.B) + (int64_t)n0 * p.ldb, p.ldb, b_rows, p.K, lds);
+  Tile::run(acc, static_cast<const T*>(p.A) + (int64_t)m0 * p.lda + k0, p.lda, a_rows,
+            static_cast<const T*>(p.B) + (int64_t)n0 * p.ldb + k0, p.ldb, b_rows, k_len, lds);
+
+  if (p.k_split > 1) {
+    float* P = p.partial + (int64_t)ks * p.M * p.N;
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+      const int col = wn * WN + ni * 32 + (lane & 31);
+      if (col >= b_rows) continue;
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wm * WM + mi * 32 + acc_row(r, lane);
+          if (row < a_rows) P[(int64_t)(m0 + row) * p.N + (n0 + col)] = acc[mi][ni][r];
+        }
+    }
+    return;
+  }
 
   OutT* C = static_cast<OutT*>(p.C);
 #pragma unroll
@@ -198,6 +290,20 @@ __global__ __launch_bounds__(512) void gemm_nt_kernel(GemmParams p) {
           *dst = cvt_out<OutT>(v);
         }
       }
+  }
+}
+
+// C[m][n] (+)= sum over splits of partial[s][m][n]
+template <typename OutT>
+__global__ void splitk_reduce_kernel(const float* __restrict__ partial, int k_split, int64_t MN, int N, OutT* C,
+                                     int64_t ldc, int accumulate) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < MN; i += (int64_t)gridDim.x * blockDim.x) {
+    float v = 0.f;
+    for (int s = 0; s < k_split; ++s) v += partial[(int64_t)s * MN + i];
+    const int64_t m = i / N, n = i - m * N;
+    OutT* dst = C + m * ldc + n;
+    if (accumulate) v += (float)*dst;
+    *dst = cvt_out<OutT>(v);
   }
 }
 
@@ -223,10 +329,10 @@ struct BwdPlan {
   int64_t ldv;        // dz / WT row stride
   int64_t chunk;      // tokens per chunk (multiple of 256 unless >= T)
   int64_t ldt;        // dzT / hidT row stride for a full chunk
-  size_t off_wt, off_hidt, off_dz, off_dzt, total;
+  size_t off_wt, off_hidt, off_dz, off_dzt, off_part, part_bytes, total;
 };
 
-static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chunk_tokens) {
+static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chunk_tokens, bool saved = false) {
   BwdPlan pl;
   pl.ldv = round_up64(V, 64);
   int64_t chunk = (chunk_tokens <= 0 || chunk_tokens >= T) ? T : round_up64(chunk_tokens, 256);
@@ -236,35 +342,51 @@ static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chun
   size_t off = 0;
   pl.off_wt = off;   off += align_up((size_t)H * pl.ldv * es, 256);
   pl.off_hidt = off; off += align_up((size_t)H * pl.ldt * es, 256);
-  pl.off_dz = off;   off += align_up((size_t)chunk * pl.ldv * es, 256);
+  pl.off_dz = off;   off += saved ? 0 : align_up((size_t)chunk * pl.ldv * es, 256);
   pl.off_dzt = off;  off += align_up((size_t)V * pl.ldt * es, 256);
+  pl.part_bytes = align_up((size_t)4 * chunk * H * sizeof(float), 256);   // split-K partials of dhidden
+  pl.off_part = off; off += pl.part_bytes;
   pl.total = off;
   return pl;
 }
 
 // Largest chunk (multiple of 256, or T itself) whose plan fits into `bytes`; 0 if none does.
-static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, size_t bytes) {
-  if (bwd_plan(T, H, V, es, T).total <= bytes) return T;
+static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, size_t bytes, bool saved) {
+  if (bwd_plan(T, H, V, es, T, saved).total <= bytes) return T;
   int64_t lo = 0, hi = T / 256;   // in units of 256 tokens
   while (lo < hi) {
     const int64_t mid = (lo + hi + 1) / 2;
-    if (bwd_plan(T, H, V, es, mid * 256).total <= bytes) lo = mid; else hi = mid - 1;
+    if (bwd_plan(T, H, V, es, mid * 256, saved).total <= bytes) lo = mid; else hi = mid - 1;
   }
   return lo * 256;
 }
 
 template <typename T>
 static int set_lds_attr(const void* fn, const char* name) {
-  using Tile = GemmTile<T, 256, 256, 2, 4>;
+  using Tile = HeadTile<T>;
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
   if (e != hipSuccess) return fail(CLGRPO_ELAUNCH, "%s: LDS attribute: %s", name, hipGetErrorString(e));
   return CLGRPO_OK;
 }
 
+// K ranges per tile that fill the 256 CUs best (1 = no split); at most what `partial_bytes` can hold.
+static int pick_k_split(int tiles, int M, int N, int K, int slab, size_t partial_bytes) {
+  int best = 1;
+  double best_eff = 0.0;
+  for (int s = 1; s <= 4; ++s) {
+    if (s > 1 && ((size_t)s * M * N * sizeof(float) > partial_bytes || K / s < 8 * slab)) break;
+    const long units = (long)tiles * s;
+    const double eff = (double)units / (double)(((units + 255) / 256) * 256);
+    if (eff > best_eff + 0.04) { best_eff = eff; best = s; }   // a split must buy more than 4 % to be worth its extra pass
+  }
+  return best;
+}
+
 template <typename T, typename OutT>
 static int launch_gemm(const void* A, int64_t lda, int M, const void* B, int64_t ldb, int N, int K, void* C,
-                       int64_t ldc, int accumulate, hipStream_t stream) {
-  using Tile = GemmTile<T, 256, 256, 2, 4>;
+                       int64_t ldc, int accumulate, hipStream_t stream, float* partial = nullptr,
+                       size_t partial_bytes = 0) {
+  using Tile = HeadTile<T>;
   static bool attr = false;
   if (!attr) {
     int rc = set_lds_attr<T>(reinterpret_cast<const void*>(&gemm_nt_kernel<T, OutT>), "gemm_nt_kernel");
@@ -276,9 +398,19 @@ static int launch_gemm(const void* A, int64_t lda, int M, const void* B, int64_t
   g.M = M; g.N = N; g.K = K;
   g.n_mt = (M + 255) / 256; g.n_nt = (N + 255) / 256;
   g.accumulate = accumulate;
-  int grid = (g.n_mt * g.n_nt + 7) / 8 * 8;
+  const int slab = Tile::kSlabK;
+  g.k_split = partial ? pick_k_split(g.n_mt * g.n_nt, M, N, K, slab, partial_bytes) : 1;
+  g.k_per_split = g.k_split > 1 ? (int)round_up64((K + g.k_split - 1) / g.k_split, slab) : K;
+  g.partial = partial;
+  int grid = (g.n_mt * g.n_nt * g.k_split + 7) / 8 * 8;
   hipLaunchKernelGGL((gemm_nt_kernel<T, OutT>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, g);
-  return check_launch("gemm_nt_kernel");
+  int rc = check_launch("gemm_nt_kernel");
+  if (rc || g.k_split == 1) return rc;
+  const int64_t MN = (int64_t)M * N;
+  int blocks = (int)((MN + 255) / 256 < 4096 ? (MN + 255) / 256 : 4096);
+  hipLaunchKernelGGL(splitk_reduce_kernel<OutT>, dim3(blocks), dim3(256), 0, stream, partial, g.k_split, MN, N,
+                     static_cast<OutT*>(C), ldc, accumulate);
+  return check_launch("splitk_reduce_kernel");
 }
 
 template <typename T>
@@ -290,17 +422,19 @@ static int launch_transpose(const T* src, int64_t ld_src, T* dst, int64_t ld_dst
 
 template <typename T>
 static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream) {
-  using Tile = GemmTile<T, 256, 256, 2, 4>;
+  using Tile = HeadTile<T>;
   const int64_t T_ = a->T, H = a->H, V = a->V;
-  const int64_t chunk = chunk_for_workspace(T_, H, V, sizeof(T), a->workspace_bytes);
+  const bool saved = a->saved_logits != nullptr;
+  const int64_t chunk = chunk_for_workspace(T_, H, V, sizeof(T), a->workspace_bytes, saved);
   if (chunk <= 0)
     return fail(CLGRPO_EWORKSPACE, "clgrpo_lmhead_bwd: workspace %zu bytes cannot hold a 256-token chunk (%zu needed)",
-                a->workspace_bytes, bwd_plan(T_, H, V, sizeof(T), 256).total);
-  const BwdPlan pl = bwd_plan(T_, H, V, sizeof(T), chunk);
+                a->workspace_bytes, bwd_plan(T_, H, V, sizeof(T), 256, saved).total);
+  const BwdPlan pl = bwd_plan(T_, H, V, sizeof(T), chunk, saved);
+  const int64_t ldz = saved ? a->ld_saved : pl.ldv;
   char* ws = static_cast<char*>(a->workspace);
-  T* wt = reinterpret_cast<T*>(ws + pl.off_wt);
+  T* wt = a->weight_t ? static_cast<T*>(a->weight_t) : reinterpret_cast<T*>(ws + pl.off_wt);
   T* hidt = reinterpret_cast<T*>(ws + pl.off_hidt);
-  T* dz = reinterpret_cast<T*>(ws + pl.off_dz);
+  T* dz_ws = reinterpret_cast<T*>(ws + pl.off_dz);
   T* dzt = reinterpret_cast<T*>(ws + pl.off_dzt);
   const T* hidden = static_cast<const T*>(a->hidden);
   const T* weight = static_cast<const T*>(a->weight);
@@ -312,7 +446,7 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream) {
     attr = true;
   }
   int rc;
-  if (a->dhidden) {
+  if (a->dhidden && !(a->weight_t && a->weight_t_ready)) {
     // WT[h][v] = W[v][h], zero for V <= v < ldv
     rc = launch_transpose<T>(weight, H, wt, pl.ldv, (int)V, (int)H, stream);
     if (rc) return rc;
@@ -320,33 +454,56 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream) {
   for (int64_t c0 = 0; c0 < T_; c0 += chunk) {
     const int64_t tc = (T_ - c0) < chunk ? (T_ - c0) : chunk;
     const int64_t ldt = round_up64(tc, 64);
-    DzParams d;
-    d.hidden = hidden + c0 * H;
-    d.weight = weight;
-    d.labels = a->labels + c0;
-    d.lse = a->lse + c0;
-    d.entropy = a->g_entropy ? a->entropy + c0 : nullptr;
-    d.g_lp = a->g_logprob + c0;
-    d.g_ent = a->g_entropy ? a->g_entropy + c0 : nullptr;
-    d.Tc = (int)tc;
-    d.ldt = (int)ldt;
-    d.H = (int)H;
-    d.V = (int)V;
-    d.ldv = (int)pl.ldv;
-    d.n_tb = (int)((ldt + 255) / 256);
-    d.n_vt = (int)((V + 255) / 256);
-    d.c = a->inv_temperature * kLog2e;
-    d.inv_temperature = a->inv_temperature;
-    d.dz = dz;
-    d.dzT = dzt;
-    int grid = (d.n_tb * d.n_vt + 7) / 8 * 8;
-    hipLaunchKernelGGL(lmhead_dz_kernel<T>, dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, d);
-    rc = check_launch("lmhead_dz_kernel");
-    if (rc) return rc;
+    T* dz = saved ? static_cast<T*>(a->saved_logits) + c0 * ldz : dz_ws;
+    if (saved) {
+      DzFromZParams q;
+      q.z = dz;
+      q.dzT = dzt;
+      q.labels = a->labels + c0;
+      q.lse = a->lse + c0;
+      q.entropy = a->g_entropy ? a->entropy + c0 : nullptr;
+      q.g_lp = a->g_logprob + c0;
+      q.g_ent = a->g_entropy ? a->g_entropy + c0 : nullptr;
+      q.Tc = (int)tc;
+      q.ldt = (int)ldt;
+      q.V = (int)V;
+      q.ldv = (int)ldz;
+      q.c = a->inv_temperature * kLog2e;
+      q.inv_temperature = a->inv_temperature;
+      dim3 grid((unsigned)((ldt + 63) / 64), (unsigned)((pl.ldv + 63) / 64));
+      hipLaunchKernelGGL(dz_from_z_kernel<T>, grid, dim3(256), 0, stream, q);
+      rc = check_launch("dz_from_z_kernel");
+      if (rc) return rc;
+    } else {
+      DzParams d;
+      d.hidden = hidden + c0 * H;
+      d.weight = weight;
+      d.labels = a->labels + c0;
+      d.lse = a->lse + c0;
+      d.entropy = a->g_entropy ? a->entropy + c0 : nullptr;
+      d.g_lp = a->g_logprob + c0;
+      d.g_ent = a->g_entropy ? a->g_entropy + c0 : nullptr;
+      d.Tc = (int)tc;
+      d.ldt = (int)ldt;
+      d.H = (int)H;
+      d.V = (int)V;
+      d.ldv = (int)pl.ldv;
+      d.n_tb = (int)((ldt + 255) / 256);
+      d.n_vt = (int)((V + 255) / 256);
+      d.c = a->inv_temperature * kLog2e;
+      d.inv_temperature = a->inv_temperature;
+      d.dz = dz;
+      d.dzT = dzt;
+      int grid = (d.n_tb * d.n_vt + 7) / 8 * 8;
+      hipLaunchKernelGGL(lmhead_dz_kernel<T>, dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, d);
+      rc = check_launch("lmhead_dz_kernel");
+      if (rc) return rc;
+    }
     if (a->dhidden) {
       // dhidden[chunk][h] = sum_v dz[t][v] WT[h][v]
-      rc = launch_gemm<T, T>(dz, pl.ldv, (int)tc, wt, pl.ldv, (int)H, (int)pl.ldv,
-                             static_cast<T*>(a->dhidden) + c0 * H, H, 0, stream);
+      rc = launch_gemm<T, T>(dz, ldz, (int)tc, wt, pl.ldv, (int)H, (int)pl.ldv,
+                             static_cast<T*>(a->dhidden) + c0 * H, H, 0, stream,
+                             reinterpret_cast<float*>(ws + pl.off_part), pl.part_bytes);
       if (rc) return rc;
     }
     if (a->dweight) {
@@ -366,9 +523,9 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream) {
 using namespace clgrpo;
 
 extern "C" size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype,
-                                                    int64_t chunk_tokens) {
+                                                    int64_t chunk_tokens, int32_t with_saved_logits) {
   if (T <= 0 || H <= 0 || V <= 0 || (dtype != CLGRPO_BF16 && dtype != CLGRPO_F32)) return 0;
-  return bwd_plan(T, H, V, dtype_bytes(dtype), chunk_tokens).total;
+  return bwd_plan(T, H, V, dtype_bytes(dtype), chunk_tokens, with_saved_logits != 0).total;
 }
 
 extern "C" int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream) {
@@ -385,6 +542,9 @@ extern "C" int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream) 
     return fail(CLGRPO_ENULL, "clgrpo_lmhead_bwd: both dhidden and dweight are NULL");
   if (!(a->inv_temperature > 0.f)) return fail(CLGRPO_EINVAL, "clgrpo_lmhead_bwd: inv_temperature must be > 0");
   CLGRPO_REQUIRE_PTR(a->workspace, "workspace");
+  if (a->saved_logits != nullptr && (a->ld_saved < round_up64(a->V, 64) || a->ld_saved % 64 != 0))
+    return fail(CLGRPO_ESHAPE, "clgrpo_lmhead_bwd: ld_saved=%lld must be a multiple of 64 and >= %lld",
+                (long long)a->ld_saved, (long long)round_up64(a->V, 64));
   hipStream_t s = static_cast<hipStream_t>(stream);
   return a->dtype == CLGRPO_BF16 ? run_bwd<__bf16>(a, s) : run_bwd<float>(a, s);
 }

@@ -25,7 +25,26 @@ struct FwdParams {
   int T, H, V;
   int n_tb, n_split, tiles_per_split, n_vt;
   float c;  // inv_temperature * log2(e)
+  void* z_out;   // optional [rows][ldz] raw logits in the input dtype
+  int64_t ldz;
+  const int32_t* z_row_map;  // optional [T]: destination row per token, < 0: not stored
+  int z_rows;                // rows of z_out; mapped rows outside [0, z_rows) are not stored
   float4* part;  // [n_split][T]: (max raw, sum 2^{(z-max) c}, sum 2^{(z-max) c} z raw, target raw)
+};
+
+template <typename T> struct Pack4;
+template <> struct Pack4<float> {
+  typedef float4 type;
+  __device__ static __forceinline__ type make(float a, float b, float c, float d) { return make_float4(a, b, c, d); }
+};
+template <> struct Pack4<__bf16> {
+  typedef uint2 type;
+  __device__ static __forceinline__ type make(float a, float b, float c, float d) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 lo = {(__bf16)a, (__bf16)b};
+    bf16x2 hi = {(__bf16)c, (__bf16)d};
+    return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+  }
 };
 
 __device__ __forceinline__ void merge_state(float& m, float& s, float& u, float om, float os,
@@ -38,9 +57,9 @@ __device__ __forceinline__ void merge_state(float& m, float& s, float& u, float 
   m = nm;
 }
 
-template <typename T>
-__global__ __launch_bounds__(512) void lmhead_fwd_kernel(FwdParams p) {
-  using Tile = GemmTile<T, kFwdBM, kFwdBN, 2, 4>;
+template <typename T, bool STORE_Z>
+__global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
+  using Tile = HeadTile<T>;
   constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
   extern __shared__ __align__(16) char lds[];
 
@@ -58,12 +77,14 @@ __global__ __launch_bounds__(512) void lmhead_fwd_kernel(FwdParams p) {
   const T* weight = static_cast<const T*>(p.weight);
   const float c = p.c;
 
-  int lab[NI];
+  int lab[NI], zrow[NI];
   float m[NI], s[NI], u[NI], zt[NI];
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
     const int tok = t0 + wn * WN + ni * 32 + (lane & 31);
     lab[ni] = (p.labels != nullptr && tok < p.T) ? (int)p.labels[tok] : -1;
+    zrow[ni] = (STORE_Z && tok < p.T) ? (p.z_row_map ? p.z_row_map[tok] : tok) : -1;
+    if (zrow[ni] >= p.z_rows) zrow[ni] = -1;
     m[ni] = -INFINITY;
     s[ni] = 0.f;
     u[ni] = 0.f;
@@ -84,6 +105,28 @@ __global__ __launch_bounds__(512) void lmhead_fwd_kernel(FwdParams p) {
         for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
     Tile::run(acc, weight + (int64_t)v0 * p.H, p.H, a_rows, hidden, p.H, b_rows, p.H, lds);
+
+    if (STORE_Z) {
+      // Raw logits for the backward: 4 consecutive vocabulary entries of one token per store.
+      // Vocabulary rows past V were read as zero rows of W, so the padding columns hold zeros.
+      T* z = static_cast<T*>(p.z_out);
+      typedef typename Pack4<T>::type P4;
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+        if (zrow[ni] >= 0) {
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int v_idx = v0 + wm * WM + mi * 32 + 8 * q + 4 * (lane >> 5);
+              if (v_idx < p.ldz)
+                *reinterpret_cast<P4*>(z + (int64_t)zrow[ni] * p.ldz + v_idx) =
+                    Pack4<T>::make(acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
+                                   acc[mi][ni][4 * q + 3]);
+            }
+        }
+      }
+    }
 
     if (a_rows == kFwdBM) {
 #pragma unroll
@@ -222,20 +265,30 @@ __global__ void lmhead_fwd_finalize_kernel(FinalizeParams p) {
   }
 }
 
+// Split of the vocabulary tiles over workgroups.  A workgroup walks ceil(n_vt / n_split) tiles for
+// one block of 256 tokens; with 256 CUs holding one workgroup each the launch takes
+// ceil(n_tb * n_split / 256) rounds, so the pick minimises rounds * tiles-per-workgroup.  At least
+// four splits when possible: the 32 workgroups of an XCD then form a 4 x 8 block sharing operands.
 static void fwd_plan(int64_t T, int64_t V, int& n_tb, int& n_vt, int& n_split, int& tiles_per_split) {
   n_tb = (int)((T + kFwdBN - 1) / kFwdBN);
   n_vt = (int)((V + kFwdBM - 1) / kFwdBM);
-  int cus = 256;
-  int want = cus / n_tb;
-  if (want < 4) want = 4;
-  if (want > n_vt) want = n_vt;
-  tiles_per_split = (n_vt + want - 1) / want;
+  const int cus = 256;
+  int best = 1;
+  long best_cost = -1;
+  for (int sp = 1; sp <= 64 && sp <= n_vt; ++sp) {
+    const int tps = (n_vt + sp - 1) / sp;
+    const int eff_sp = (n_vt + tps - 1) / tps;
+    const long rounds = ((long)n_tb * eff_sp + cus - 1) / cus;
+    long cost = rounds * tps * 16 + (sp < 4 ? 8 : 0) + eff_sp / 8;   // small penalties break ties
+    if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = sp; }
+  }
+  tiles_per_split = (n_vt + best - 1) / best;
   n_split = (n_vt + tiles_per_split - 1) / tiles_per_split;
 }
 
-template <typename T>
+template <typename T, bool STORE_Z>
 static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream) {
-  using Tile = GemmTile<T, kFwdBM, kFwdBN, 2, 4>;
+  using Tile = HeadTile<T>;
   FwdParams p;
   p.hidden = a->hidden;
   p.weight = a->weight;
@@ -246,16 +299,20 @@ static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream) {
   fwd_plan(a->T, a->V, p.n_tb, p.n_vt, p.n_split, p.tiles_per_split);
   p.c = a->inv_temperature * kLog2e;
   p.part = static_cast<float4*>(a->workspace);
+  p.z_out = a->saved_logits;
+  p.ldz = a->ld_saved;
+  p.z_row_map = a->saved_row_map;
+  p.z_rows = (int)a->saved_rows;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&lmhead_fwd_kernel<T>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&lmhead_fwd_kernel<T, STORE_Z>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
     if (e != hipSuccess) return fail(CLGRPO_ELAUNCH, "lmhead_fwd: LDS attribute: %s", hipGetErrorString(e));
     attr_set = true;
   }
   int grid = p.n_tb * p.n_split;
   grid = (grid + 7) / 8 * 8;
-  hipLaunchKernelGGL(lmhead_fwd_kernel<T>, dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, p);
+  hipLaunchKernelGGL((lmhead_fwd_kernel<T, STORE_Z>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, p);
   int rc = check_launch("lmhead_fwd_kernel");
   if (rc) return rc;
   FinalizeParams f;
@@ -288,6 +345,8 @@ int validate_head_shape(const char* who, int64_t T, int64_t H, int64_t V, int32_
 
 using namespace clgrpo;
 
+extern "C" int64_t clgrpo_saved_logits_ld(int64_t V) { return V <= 0 ? 0 : round_up64(V, 64); }
+
 extern "C" size_t clgrpo_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype) {
   (void)H;
   (void)dtype;
@@ -310,6 +369,13 @@ extern "C" int clgrpo_lmhead_fwd(const clgrpo_lmhead_fwd_args* a, void* stream) 
   const size_t need = clgrpo_lmhead_fwd_workspace_bytes(a->T, a->H, a->V, a->dtype);
   if (a->workspace_bytes < need)
     return fail(CLGRPO_EWORKSPACE, "clgrpo_lmhead_fwd: workspace %zu < %zu bytes", a->workspace_bytes, need);
+  if (a->saved_logits != nullptr && (a->ld_saved < clgrpo_saved_logits_ld(a->V) || a->ld_saved % 64 != 0))
+    return fail(CLGRPO_ESHAPE, "clgrpo_lmhead_fwd: ld_saved=%lld must be a multiple of 64 and >= %lld",
+                (long long)a->ld_saved, (long long)clgrpo_saved_logits_ld(a->V));
+  if (a->saved_logits != nullptr && (a->saved_rows <= 0 || a->saved_rows >= (1LL << 31)))
+    return fail(CLGRPO_EINVAL, "clgrpo_lmhead_fwd: saved_rows=%lld", (long long)a->saved_rows);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return a->dtype == CLGRPO_BF16 ? launch_fwd<__bf16>(a, s) : launch_fwd<float>(a, s);
+  if (a->saved_logits != nullptr)
+    return a->dtype == CLGRPO_BF16 ? launch_fwd<__bf16, true>(a, s) : launch_fwd<float, true>(a, s);
+  return a->dtype == CLGRPO_BF16 ? launch_fwd<__bf16, false>(a, s) : launch_fwd<float, false>(a, s);
 }

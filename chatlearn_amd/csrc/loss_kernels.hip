@@ -19,7 +19,7 @@ constexpr int kNumSums = 8;
 
 struct LossParams {
   int mode;
-  int64_t n, B, S;
+  int64_t n, B, S, token_offset;
   const int32_t* cu_seqlens;
   const float* logprob;
   const float* old_logprob;
@@ -45,8 +45,9 @@ struct LossParams {
 
 __device__ __forceinline__ int seq_of_token(const LossParams& p, int64_t i) {
   if (p.cu_seqlens == nullptr) return (int)(i / p.S);
+  i += p.token_offset;
   // largest b with cu_seqlens[b] <= i; tokens at or past cu_seqlens[B] belong to no sequence
-  if (i >= p.cu_seqlens[p.B]) return -1;
+  if (i >= p.cu_seqlens[p.B] || i < p.cu_seqlens[0]) return -1;
   int lo = 0, hi = (int)p.B;  // invariant: cu[lo] <= i < cu[hi]
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -66,8 +67,13 @@ __device__ __forceinline__ double wave_sum(double v) {
 __global__ __launch_bounds__(kLossThreads) void gspo_seq_mean_kernel(LossParams p) {
   const int b = blockIdx.x;
   int64_t begin, end;
-  if (p.cu_seqlens) { begin = p.cu_seqlens[b]; end = p.cu_seqlens[b + 1]; }
-  else { begin = (int64_t)b * p.S; end = begin + p.S; }
+  if (p.cu_seqlens) {
+    // positions relative to this call's first token; a sequence outside the window contributes nothing
+    begin = (int64_t)p.cu_seqlens[b] - p.token_offset;
+    end = (int64_t)p.cu_seqlens[b + 1] - p.token_offset;
+    if (begin < 0) begin = 0;
+    if (end > p.n) end = p.n;
+  } else { begin = (int64_t)b * p.S; end = begin + p.S; }
   double num = 0.0, den = 0.0;
   for (int64_t i = begin + threadIdx.x; i < end; i += kLossThreads) {
     const int mk = p.loss_mask ? p.loss_mask[i] : 1;
@@ -226,6 +232,7 @@ extern "C" int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream
     return fail(CLGRPO_EINVAL, "clgrpo_policy_loss: mode %d", a->mode);
   if (a->compute_dtype != CLGRPO_F32 && a->compute_dtype != CLGRPO_F64)
     return fail(CLGRPO_EDTYPE, "clgrpo_policy_loss: compute_dtype %d", a->compute_dtype);
+  if (a->token_offset < 0) return fail(CLGRPO_EINVAL, "clgrpo_policy_loss: token_offset=%lld", (long long)a->token_offset);
   if (a->n < 0 || a->B <= 0) return fail(CLGRPO_EINVAL, "clgrpo_policy_loss: n=%lld B=%lld", (long long)a->n, (long long)a->B);
   if (a->cu_seqlens == nullptr) {
     if (a->S <= 0 || a->B * a->S != a->n)
@@ -248,6 +255,7 @@ extern "C" int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream
   LossParams p;
   p.mode = a->mode;
   p.n = a->n; p.B = a->B; p.S = a->S;
+  p.token_offset = a->cu_seqlens ? a->token_offset : 0;
   p.cu_seqlens = a->cu_seqlens;
   p.logprob = a->logprob; p.old_logprob = a->old_logprob; p.ref_logprob = a->ref_logprob;
   p.entropy = a->entropy; p.loss_mask = a->loss_mask; p.advantages = a->advantages;

@@ -7,9 +7,10 @@ states and lm_head.weight, without the [T, V] logits tensor.
 autograd-aware, so ``total_loss.backward()`` (policy_trainer.py:286) reaches
 ``hidden`` and ``weight`` through the fused backward kernels.
 
-``grpo_head_step`` does a whole micro-batch of the head in three launches
-groups - fused forward, fused loss (+ upstream gradients), fused backward -
-for callers that own the training loop.
+``grpo_head_step`` does a whole micro-batch of the head - fused forward, fused
+loss (+ upstream gradients), fused backward - for callers that own the training
+loop; it walks the micro-batch in token chunks and lets the backward reuse the
+chunk's logits instead of recomputing them.
 """
 from typing import Optional
 
@@ -72,41 +73,147 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     return lp, ent
 
 
+def _token_chunks(T, chunk_tokens, seq_bounds):
+    """[lo, hi) token ranges of about ``chunk_tokens`` tokens.  With ``seq_bounds`` (the host copy of
+    cu_seqlens) every range ends on a sequence boundary, growing past the target where one
+    sequence is longer than it."""
+    if chunk_tokens is None or chunk_tokens >= T:
+        return [(0, T)]
+    if seq_bounds is None:
+        return [(lo, min(T, lo + chunk_tokens)) for lo in range(0, T, chunk_tokens)]
+    out, lo = [], 0
+    for b in range(1, len(seq_bounds)):
+        nxt = seq_bounds[b + 1] if b + 1 < len(seq_bounds) else None
+        if nxt is None or nxt - lo > chunk_tokens:
+            if seq_bounds[b] > lo:
+                out.append((lo, seq_bounds[b]))
+                lo = seq_bounds[b]
+    if lo < T:
+        out.append((lo, T))
+    return out
+
+
 def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages, cu_seqlens, loss_mask, *,
                    n_tokens_total: float, fsdp_size: int = 1, use_group_sequence_policy=False,
                    pos_clip_ratio=0.2, neg_clip_ratio=0.2, diff_clip_ratio=10, final_clip_ratio=3,
                    kl_coef=0.0, entropy_coef=0.0, temperature=1.0, dweight: Optional[torch.Tensor] = None,
-                   accumulate_dweight=False, need_dhidden=True, check_flags=True):
+                   accumulate_dweight=False, need_dhidden=True, check_flags=True,
+                   keep_logits_chunk: Optional[int] = 8192, cu_seqlens_host=None, skip_masked_rows=True,
+                   stage_hook=None):
     """Forward + loss + backward of the head for one packed micro-batch, no autograd graph.
 
     Mirrors policy_trainer.py:216-286 on packed rows: returns a dict with the
     per-token ``logprob``/``entropy``, the loss scalars ``pg_loss_mean``,
     ``kl_loss_mean``, ``entropy_loss_mean``, ``total_loss`` (device fp64 scalars),
     ``dhidden`` and ``dweight``.  ``advantages`` is a device tensor [B].
+
+    ``keep_logits_chunk``: the micro-batch is walked in chunks of about this many tokens; within
+    a chunk the forward keeps its raw logits (one [chunk, V] buffer in the input dtype, reused
+    chunk after chunk) so the backward does not recompute them.  ``None`` keeps nothing: the
+    backward then recomputes the logit tiles from ``hidden`` and ``weight``.  The sequence-level
+    loss needs chunks that end on sequence boundaries, so it reads ``cu_seqlens_host`` (or copies
+    ``cu_seqlens`` to the host once).
+
+    ``skip_masked_rows`` (only with kept logits and a loss mask): rows whose mask is zero have an
+    exactly zero upstream gradient, so the backward runs on the compacted set of the other rows
+    (their dhidden rows are zero); ``rows_projected_bwd`` in the result counts the rows it ran on.
+
+    ``stage_hook(name)`` is called on the host at "forward", "loss", "backward", "end" boundaries
+    of every chunk (a benchmark records stream events there).
     """
-    lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, temperature, need_entropy=True)
+    hook = stage_hook or (lambda name: None)
+    T = hidden.shape[0]
+    V = weight.shape[0]
     scale = float(fsdp_size) / float(n_tokens_total)
-    res = ops.policy_loss(
-        lp, old_logprob, advantages, mode=LOSS_GSPO if use_group_sequence_policy else LOSS_GRPO,
-        cu_seqlens=cu_seqlens, ref_logprob=ref_logprob, entropy=ent, loss_mask=loss_mask,
-        diff_clip_ratio=diff_clip_ratio, pos_clip_ratio=pos_clip_ratio, neg_clip_ratio=neg_clip_ratio,
-        final_clip_ratio=final_clip_ratio, kl_coef=kl_coef if kl_coef > 0 else 0.0,
-        entropy_coef=entropy_coef if entropy_coef > 0 else 0.0, grad_scale=scale, want_dloss=False,
-        want_upstream=True)
-    dh, dw = ops.lmhead_backward(hidden, weight, labels, lse, ent, res.g_logprob, res.g_entropy, temperature,
-                                 need_dhidden=need_dhidden, need_dweight=True, dweight=dweight,
-                                 accumulate_dweight=accumulate_dweight)
+    mode = LOSS_GSPO if use_group_sequence_policy else LOSS_GRPO
+    bounds = None
+    if keep_logits_chunk is not None and keep_logits_chunk < T and use_group_sequence_policy:
+        bounds = list(cu_seqlens_host) if cu_seqlens_host is not None else cu_seqlens.tolist()
+    chunks = _token_chunks(T, keep_logits_chunk, bounds)
+    zbuf = None
+    if keep_logits_chunk is not None:
+        zbuf = ops.saved_logits_buffer(max(hi - lo for lo, hi in chunks), V, hidden.dtype, hidden.device)
+    f = dict(dtype=torch.float32, device=hidden.device)
+    lp_all, ent_all, lse_all, glp_all = (torch.empty(T, **f) for _ in range(4))
+    loss_all = torch.empty(T, dtype=advantages.dtype, device=hidden.device)
+    kl_all = torch.empty(T, **f) if ref_logprob is not None else None
+    dh_all = torch.empty_like(hidden) if need_dhidden else None
+    sums = torch.zeros(8, dtype=torch.float64, device=hidden.device)
+    flags = torch.zeros(1, dtype=torch.int32, device=hidden.device)
+    dw = dweight
+    acc_dw = accumulate_dweight
+    rows_projected_bwd = 0
+    wt = ops.weight_t_buffer(weight) if (need_dhidden and len(chunks) > 1) else None
+    wt_ready = False
+    kl_c = kl_coef if kl_coef > 0 else 0.0
+    en_c = entropy_coef if entropy_coef > 0 else 0.0
+    for lo, hi in chunks:
+        sl = slice(lo, hi)
+        n = hi - lo
+        live = row_map = None
+        if zbuf is not None and loss_mask is not None and skip_masked_rows:
+            # Rows whose loss mask is zero get a zero upstream gradient whatever the logits are:
+            # keep logits only for the others and run the backward on that compact set of rows.
+            live, _, _, _ = ops.unpad_indices(loss_mask[sl].reshape(1, n))
+            row_map = torch.full((n,), -1, dtype=torch.int32, device=hidden.device)
+            row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
+        hook("forward")
+        lp, ent, _, lse = ops.lmhead_forward(hidden[sl], weight, labels[sl], temperature, need_entropy=True,
+                                             saved_logits=zbuf, saved_row_map=row_map)
+        hook("loss")
+        res = ops.policy_loss(
+            lp, old_logprob[sl], advantages, mode=mode, cu_seqlens=cu_seqlens,
+            ref_logprob=None if ref_logprob is None else ref_logprob[sl], entropy=ent,
+            loss_mask=None if loss_mask is None else loss_mask[sl], diff_clip_ratio=diff_clip_ratio,
+            pos_clip_ratio=pos_clip_ratio, neg_clip_ratio=neg_clip_ratio, final_clip_ratio=final_clip_ratio,
+            kl_coef=kl_c, entropy_coef=en_c, grad_scale=scale, want_dloss=False, want_upstream=True,
+            token_offset=lo)
+        hook("backward")
+        if live is None:
+            dh, dw = ops.lmhead_backward(hidden[sl], weight, labels[sl], lse, ent, res.g_logprob, res.g_entropy,
+                                         temperature, need_dhidden=need_dhidden, need_dweight=True, dweight=dw,
+                                         accumulate_dweight=acc_dw, saved_logits=zbuf, weight_t=wt,
+                                         weight_t_ready=wt_ready)
+            wt_ready = True
+        elif live.numel() == 0:
+            dh = torch.zeros_like(hidden[sl]) if need_dhidden else None
+            if not acc_dw:
+                dw = torch.zeros(V, hidden.shape[1], dtype=torch.float32, device=hidden.device) if dw is None \
+                    else dw.zero_()
+        else:
+            pick = lambda x: None if x is None else ops.gather_rows(x.reshape(n, -1), live).reshape(-1)
+            dh_c, dw = ops.lmhead_backward(
+                ops.gather_rows(hidden[sl], live), weight, pick(labels[sl]), pick(lse), pick(ent),
+                pick(res.g_logprob), pick(res.g_entropy), temperature, need_dhidden=need_dhidden,
+                need_dweight=True, dweight=dw, accumulate_dweight=acc_dw, saved_logits=zbuf, weight_t=wt,
+                weight_t_ready=wt_ready)
+            wt_ready = True
+            dh = ops.scatter_rows(dh_c, live, n) if need_dhidden else None
+            rows_projected_bwd += int(live.numel()) - n
+        rows_projected_bwd += n
+        hook("end")
+        acc_dw = True
+        lp_all[sl], ent_all[sl], lse_all[sl], glp_all[sl], loss_all[sl] = lp, ent, lse, res.g_logprob, res.loss
+        if kl_all is not None:
+            kl_all[sl] = res.kl
+        if need_dhidden:
+            dh_all[sl] = dh
+        sums += res.sums
+        flags |= res.flags
     if check_flags:
-        res.raise_on_flags()
-    pg = res.sums[0] * scale
-    kl = res.sums[1] * scale
-    en = res.sums[2] * scale
+        fl = int(flags.item())
+        assert not fl & 1, "pg loss is nan"
+        assert not fl & 2, "kl loss ratio has inf values"
+        assert not fl & 4, "kl loss ratio has nan values"
+    pg = sums[0] * scale
+    kl = sums[1] * scale
+    en = sums[2] * scale
     total = pg
     if entropy_coef > 0:
         total = total - entropy_coef * en
     if kl_coef > 0:
         total = total + kl_coef * kl
-    return {"logprob": lp, "entropy": ent, "lse": lse, "pg_loss_mean": pg, "kl_loss_mean": kl,
-            "entropy_loss_mean": en, "total_loss": total, "num_masked": res.sums[3],
-            "per_token_loss": res.loss, "per_token_kl": res.kl, "dhidden": dh, "dweight": dw,
-            "g_logprob": res.g_logprob}
+    return {"logprob": lp_all, "entropy": ent_all, "lse": lse_all, "pg_loss_mean": pg, "kl_loss_mean": kl,
+            "entropy_loss_mean": en, "total_loss": total, "num_masked": sums[3],
+            "per_token_loss": loss_all, "per_token_kl": kl_all, "dhidden": dh_all, "dweight": dw,
+            "g_logprob": glp_all, "rows_projected_bwd": rows_projected_bwd}

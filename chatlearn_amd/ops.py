@@ -45,10 +45,25 @@ def _stream(t: torch.Tensor):
 
 # --------------------------------------------------------------------------- fused lm_head
 
+def saved_logits_buffer(T: int, V: int, dtype, device) -> torch.Tensor:
+    """An (uninitialised) [T, ld] buffer the forward can store raw logits in for the backward."""
+    return torch.empty(T, _lib.lib().clgrpo_saved_logits_ld(V), dtype=dtype, device=device)
+
+
+def weight_t_buffer(weight: torch.Tensor) -> torch.Tensor:
+    """An (uninitialised) [H, ld] buffer for W^T that ``lmhead_backward`` can fill once and reuse."""
+    V, H = weight.shape
+    return torch.empty(H, _lib.lib().clgrpo_saved_logits_ld(V), dtype=weight.dtype, device=weight.device)
+
+
 def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[torch.Tensor],
-                   temperature: float = 1.0, need_entropy: bool = True
+                   temperature: float = 1.0, need_entropy: bool = True,
+                   saved_logits: Optional[torch.Tensor] = None, saved_row_map: Optional[torch.Tensor] = None
                    ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], torch.Tensor, torch.Tensor]:
-    """(logprob, entropy, rowmax, lse), each fp32 [T]; logits are never materialised."""
+    """(logprob, entropy, rowmax, lse), each fp32 [T].  Logits are not materialised unless the caller
+    hands in ``saved_logits`` (from ``saved_logits_buffer``) for these T rows, which a following
+    ``lmhead_backward`` of the same rows consumes instead of recomputing them.  ``saved_row_map``
+    (int32 [T]) sends token t's logits to row ``map[t]`` of the buffer, or nowhere if negative."""
     hidden = _dev(hidden, "hidden")
     weight = _dev(weight, "weight", hidden.dtype)
     if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
@@ -69,8 +84,22 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
         return logprob, entropy, rowmax, lse
     ws_bytes = _lib.lib().clgrpo_lmhead_fwd_workspace_bytes(T, H, V, dt)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=hidden.device)
+    ld_saved = 0
+    if saved_logits is not None:
+        saved_logits = _dev(saved_logits, "saved_logits", hidden.dtype)
+        if saved_logits.dim() != 2 or not saved_logits.is_contiguous():
+            raise ValueError("saved_logits must be a contiguous [rows, ld] tensor")
+        if saved_row_map is None and saved_logits.shape[0] < T:
+            raise ValueError("saved_logits needs at least T rows")
+        ld_saved = saved_logits.shape[1]
+        if saved_row_map is not None:
+            saved_row_map = _dev(saved_row_map, "saved_row_map", torch.int32)
+            if saved_row_map.numel() != T:
+                raise ValueError("saved_row_map must have T elements")
     a = _lib.LmheadFwdArgs(_ptr(hidden), _ptr(weight), _ptr(labels), T, H, V, dt, 1.0 / float(temperature),
-                           _ptr(logprob), _ptr(entropy), _ptr(rowmax), _ptr(lse), _ptr(ws), ws.numel())
+                           _ptr(logprob), _ptr(entropy), _ptr(rowmax), _ptr(lse), _ptr(ws), ws.numel(),
+                           _ptr(saved_logits), ld_saved, _ptr(saved_row_map) if saved_logits is not None else None,
+                           saved_logits.shape[0] if saved_logits is not None else 0)
     _lib.call("clgrpo_lmhead_fwd", a, _stream(hidden))
     return logprob, entropy, rowmax, lse
 
@@ -78,9 +107,14 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
 def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=None, temperature=1.0,
                     need_dhidden=True, need_dweight=True, dweight: Optional[torch.Tensor] = None,
                     accumulate_dweight=False, chunk_tokens: Optional[int] = None,
-                    max_workspace_bytes: int = DEFAULT_BWD_WORKSPACE_BYTES):
+                    max_workspace_bytes: int = DEFAULT_BWD_WORKSPACE_BYTES,
+                    saved_logits: Optional[torch.Tensor] = None, weight_t: Optional[torch.Tensor] = None,
+                    weight_t_ready: bool = False):
     """(dhidden [T,H] in hidden's dtype, dweight [V,H] fp32).  ``dweight`` may be a caller
-    buffer (e.g. the fp32 main-grad) that is overwritten or, with ``accumulate_dweight``, added to."""
+    buffer (e.g. the fp32 main-grad) that is overwritten or, with ``accumulate_dweight``, added to.
+    ``saved_logits``: the buffer the forward of these rows filled; it is overwritten with d(logits).
+    ``weight_t`` (from ``weight_t_buffer``) keeps W^T between calls that share the weight; pass
+    ``weight_t_ready=True`` once a call has filled it."""
     hidden = _dev(hidden, "hidden")
     weight = _dev(weight, "weight", hidden.dtype)
     labels = _dev(labels, "labels", torch.int64)
@@ -113,15 +147,27 @@ def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=N
             dweight.zero_()
         return dhidden, dweight
     L = _lib.lib()
+    ld_saved, has_saved = 0, 0
+    if saved_logits is not None:
+        saved_logits = _dev(saved_logits, "saved_logits", hidden.dtype)
+        if saved_logits.dim() != 2 or saved_logits.shape[0] < T or not saved_logits.is_contiguous():
+            raise ValueError("saved_logits must be a contiguous [>=T, ld] tensor")
+        ld_saved, has_saved = saved_logits.shape[1], 1
+    if weight_t is not None:
+        weight_t = _dev(weight_t, "weight_t", hidden.dtype)
+        if tuple(weight_t.shape) != (H, L.clgrpo_saved_logits_ld(V)) or not weight_t.is_contiguous():
+            raise ValueError("weight_t must come from weight_t_buffer(weight)")
     if chunk_tokens is None:
         chunk_tokens = T
-        while chunk_tokens > 256 and L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens) > max_workspace_bytes:
+        while chunk_tokens > 256 and \
+                L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens, has_saved) > max_workspace_bytes:
             chunk_tokens = max(256, (chunk_tokens // 2 + 255) // 256 * 256)
-    ws_bytes = L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens)
+    ws_bytes = L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens, has_saved)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hidden.device)
     a = _lib.LmheadBwdArgs(_ptr(hidden), _ptr(weight), _ptr(labels), _ptr(lse), _ptr(entropy), _ptr(g_logprob),
                            _ptr(g_entropy), T, H, V, dt, 1.0 / float(temperature), _ptr(dhidden), _ptr(dweight),
-                           1 if accumulate_dweight else 0, _ptr(ws), ws.numel())
+                           1 if accumulate_dweight else 0, _ptr(ws), ws.numel(), _ptr(saved_logits), ld_saved,
+                           _ptr(weight_t), 1 if (weight_t is not None and weight_t_ready) else 0)
     _lib.call("clgrpo_lmhead_bwd", a, _stream(hidden))
     return dhidden, dweight
 
@@ -189,7 +235,7 @@ class PolicyLossResult:
 def policy_loss(logprob, old_logprob, advantages, *, mode=LOSS_GRPO, cu_seqlens=None, ref_logprob=None,
                 entropy=None, loss_mask=None, diff_clip_ratio=10, pos_clip_ratio=0.2, neg_clip_ratio=0.2,
                 final_clip_ratio=3.0, kl_coef=0.0, entropy_coef=0.0, grad_scale=1.0, want_dloss=True,
-                want_kl=None, want_flags3=False, want_upstream=False) -> PolicyLossResult:
+                want_kl=None, want_flags3=False, want_upstream=False, token_offset=0) -> PolicyLossResult:
     """logprob/old/ref/entropy fp32, either [B,S] (padded) or flat [n] with ``cu_seqlens`` int32 [B+1];
     ``advantages`` a device tensor [B], fp32 or fp64 (sets the dtype of the loss)."""
     logprob = _dev(logprob, "logprob", torch.float32)
@@ -249,7 +295,8 @@ def policy_loss(logprob, old_logprob, advantages, *, mode=LOSS_GRPO, cu_seqlens=
                             float(pos_clip_ratio), float(neg_clip_ratio), float(final_clip_ratio), float(kl_coef),
                             float(entropy_coef), float(grad_scale), _ptr(r.loss), _ptr(r.dloss), _ptr(r.kl),
                             _ptr(r.is_positive_clipped), _ptr(r.is_negative_clipped), _ptr(r.is_clipped),
-                            _ptr(r.g_logprob), _ptr(r.g_entropy), _ptr(r.sums), _ptr(r.flags), _ptr(ws), ws.numel())
+                            _ptr(r.g_logprob), _ptr(r.g_entropy), _ptr(r.sums), _ptr(r.flags), _ptr(ws), ws.numel(),
+                            int(token_offset))
     _lib.call("clgrpo_policy_loss", a, _stream(logprob))
     return r
 

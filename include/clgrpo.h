@@ -58,7 +58,19 @@ typedef struct {
   float* lse;              /* [T] out, fp32 (logsumexp_v z); required */
   void* workspace;
   size_t workspace_bytes;
+  void* saved_logits;      /* optional out [T][ld_saved] in `dtype`: the raw logits hidden.W^T (before the
+                              temperature), for a later clgrpo_lmhead_bwd of the SAME T rows that then skips
+                              the recomputation.  NULL: nothing is stored.  Callers bound its size by
+                              processing a micro-batch in token chunks. */
+  int64_t ld_saved;        /* row stride in elements, a multiple of 64, >= clgrpo_saved_logits_ld(V) */
+  const int32_t* saved_row_map; /* optional [T]: row of saved_logits that receives token t's logits, or a
+                              negative value to store nothing for t (tokens whose upstream gradient is
+                              known to be zero, e.g. masked-out prompt positions).  NULL: row t. */
+  int64_t saved_rows;      /* rows of saved_logits; a mapped row outside [0, saved_rows) is not stored */
 } clgrpo_lmhead_fwd_args;
+
+/* Row stride (elements) the saved-logits buffer must have: V rounded up to 64. */
+int64_t clgrpo_saved_logits_ld(int64_t V);
 
 size_t clgrpo_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype);
 int clgrpo_lmhead_fwd(const clgrpo_lmhead_fwd_args* a, void* stream);
@@ -87,11 +99,18 @@ typedef struct {
   int32_t accumulate_dweight; /* nonzero: dweight += ; zero: dweight = */
   void* workspace;
   size_t workspace_bytes;   /* sets the token chunk: see clgrpo_lmhead_bwd_workspace_bytes */
+  void* saved_logits;       /* optional in/out [T][ld_saved]: logits stored by clgrpo_lmhead_fwd for these
+                               rows.  Overwritten in place with d(logits); the recomputation is skipped. */
+  int64_t ld_saved;
+  void* weight_t;           /* optional [H][clgrpo_saved_logits_ld(V)] in `dtype`: caller-kept W^T, so that
+                               several calls with the same weight (token chunks of one step) build it once */
+  int32_t weight_t_ready;   /* zero: this call fills weight_t; nonzero: it already holds W^T */
 } clgrpo_lmhead_bwd_args;
 
-/* Bytes needed to process `chunk_tokens` tokens at a time (chunk_tokens <= 0: all T at once). */
+/* Bytes needed to process `chunk_tokens` tokens at a time (chunk_tokens <= 0: all T at once);
+ * with_saved_logits != 0: the d(logits) buffer is the caller's saved_logits, not part of the workspace. */
 size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype,
-                                         int64_t chunk_tokens);
+                                         int64_t chunk_tokens, int32_t with_saved_logits);
 int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream);
 
 /* ------------------------------------------------------------------ *
@@ -165,6 +184,8 @@ typedef struct {
   int32_t* flags;            /* [1] out: bit0 loss has NaN, bit1 exp(k) has Inf, bit2 exp(k) has NaN */
   void* workspace;
   size_t workspace_bytes;
+  int64_t token_offset;      /* packed layout: position of token 0 of this call inside the row that
+                                cu_seqlens describes (lets a caller walk a micro-batch in token chunks) */
 } clgrpo_policy_loss_args;
 
 size_t clgrpo_policy_loss_workspace_bytes(int64_t n, int64_t B);

@@ -19,7 +19,7 @@ def _declared():
 
 def test_every_declared_symbol_is_exported_and_bound(lib):
     names = _declared()
-    assert len(names) >= 18
+    assert len(names) >= 19
     for n in names:
         assert hasattr(lib, n), f"{n} declared in clgrpo.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
@@ -29,8 +29,8 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 
 def test_struct_sizes_match_header_layout():
     # 64-bit pointers and int64 fields, natural alignment
-    assert C.sizeof(_lib.LmheadFwdArgs) == 3 * 8 + 3 * 8 + 4 + 4 + 4 * 8 + 8 + 8
-    assert C.sizeof(_lib.LmheadBwdArgs) == 7 * 8 + 3 * 8 + 4 + 4 + 2 * 8 + 8 + 8 + 8
+    assert C.sizeof(_lib.LmheadFwdArgs) == 3 * 8 + 3 * 8 + 4 + 4 + 4 * 8 + 8 + 8 + 8 + 8 + 8 + 8
+    assert C.sizeof(_lib.LmheadBwdArgs) == 7 * 8 + 3 * 8 + 4 + 4 + 2 * 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8
     assert C.sizeof(_lib.RowsArgs) == 6 * 8
 
 
@@ -52,9 +52,11 @@ def test_validation_before_launch(lib):
     b = _lib.LmheadBwdArgs()
     b.T, b.H, b.V, b.dtype = 8, 128, 50, _lib.F32
     assert lib.clgrpo_lmhead_bwd(C.byref(b), None) == -4
-    full = lib.clgrpo_lmhead_bwd_workspace_bytes(1024, 128, 1000, _lib.BF16, 0)
-    half = lib.clgrpo_lmhead_bwd_workspace_bytes(1024, 128, 1000, _lib.BF16, 512)
-    assert 0 < half < full
+    full = lib.clgrpo_lmhead_bwd_workspace_bytes(1024, 128, 1000, _lib.BF16, 0, 0)
+    half = lib.clgrpo_lmhead_bwd_workspace_bytes(1024, 128, 1000, _lib.BF16, 512, 0)
+    saved = lib.clgrpo_lmhead_bwd_workspace_bytes(1024, 128, 1000, _lib.BF16, 0, 1)
+    assert 0 < half < full and saved == full - 1024 * 1024 * 2   # minus the [T][ld] d(logits) buffer
+    assert lib.clgrpo_saved_logits_ld(151936) == 151936 and lib.clgrpo_saved_logits_ld(1000) == 1024
     p = _lib.PolicyLossArgs()
     p.mode = 5
     assert lib.clgrpo_policy_loss(C.byref(p), None) == -1

@@ -1,0 +1,98 @@
+"""Whole head step (fused forward + loss + backward) on packed micro-batches against the
+oracle's restatement of the reference's loop body; kept-logits and recompute paths, chunking."""
+import pytest
+import torch
+
+from chatlearn_amd import synthetic
+from tests.util import assert_close_rel, oracle_head_step
+
+pytestmark = pytest.mark.gpu
+
+
+def _workload(name, dev, **kw):
+    cfg = synthetic.scaled(synthetic.CONFIGS[name], **kw)
+    gen = synthetic.generator_for(cfg)
+    samples = synthetic.fill_microbatch(cfg, synthetic.sample_population(cfg, gen))
+    cu, mask = synthetic.packed_layout(samples)
+    T = int(cu[-1])
+    hidden, weight, labels = synthetic.make_head_tensors(cfg, T, gen)
+    from oracle import softmax_stats as osm
+    lp64, *_ = osm.fused_head_forward(hidden, weight, labels, cfg.temperature)
+    old, ref = synthetic.noisy_logprobs(lp64, gen, 0.05 if cfg.loss != "gspo" else 0.002, 0.1)
+    from oracle import advantage as oadv
+    pop = [dict(s) for s in samples]
+    oadv.AdvantageComputer(cfg.group)([oadv._Buffer(pop)])
+    adv = torch.tensor([float(s["advantages"]) for s in pop], dtype=torch.float32)
+    return cfg, samples, cu, mask, T, hidden, weight, labels, old, ref, adv
+
+
+CASES = [
+    # the five benchmark recipes at sizes the CPU oracle finishes in seconds
+    ("c1", dict(H=256, V=6000)),
+    ("c2", dict(H=512, V=5000, T=2048, n_prompts=4, group=4, prompt_range=(16, 64), response_range=(32, 256))),
+    ("c3", dict(H=256, V=5000, T=3000, n_prompts=2, group=8, response_range=(64, 512))),
+    ("c5", dict(H=512, V=4040, T=2048, response_range=(128, 512))),
+]
+
+
+@pytest.mark.parametrize("name,kw", CASES, ids=[c[0] for c in CASES])
+@pytest.mark.parametrize("keep", [None, 512, 100000], ids=["recompute", "chunked-keep", "keep-all"])
+def test_head_step_matches_oracle(dev, name, kw, keep):
+    from chatlearn_amd.fused import grpo_head_step
+    cfg, samples, cu, mask, T, hidden, weight, labels, old, ref, adv = _workload(name, dev, **kw)
+    n_tok = float(mask.sum())
+    gspo = cfg.loss == "gspo"
+    want = oracle_head_step(hidden, weight, labels, old, ref, adv, cu, mask, n_tok=n_tok, temperature=cfg.temperature,
+                            kl_coef=cfg.kl_coef, entropy_coef=cfg.entropy_coef, gspo=gspo, pos=cfg.pos_clip_ratio,
+                            neg=cfg.neg_clip_ratio, final=cfg.final_clip_ratio)
+    d = lambda x: x.to(dev)
+    got = grpo_head_step(d(hidden), d(weight), d(labels), d(old), d(ref), d(adv), d(cu), d(mask), n_tokens_total=n_tok,
+                         use_group_sequence_policy=gspo, pos_clip_ratio=cfg.pos_clip_ratio,
+                         neg_clip_ratio=cfg.neg_clip_ratio, final_clip_ratio=cfg.final_clip_ratio, kl_coef=cfg.kl_coef,
+                         entropy_coef=cfg.entropy_coef, temperature=cfg.temperature, keep_logits_chunk=keep,
+                         cu_seqlens_host=cu.tolist())
+    rt = 1e-5 if cfg.dtype == torch.float32 else 1e-2
+    assert_close_rel(got["logprob"], want["logprob"], rt, "logprob")
+    assert_close_rel(got["entropy"], want["entropy"], rt, "entropy")
+    assert float(got["total_loss"]) == pytest.approx(float(want["total_loss"]), rel=rt, abs=rt * 1e-3)
+    assert float(got["pg_loss_mean"]) == pytest.approx(float(want["parts"]["pg_loss_mean"]), rel=rt, abs=rt * 1e-3)
+    assert float(got["kl_loss_mean"]) == pytest.approx(float(want["parts"]["kl_loss_mean"]), rel=rt, abs=rt * 1e-3)
+    # GSPO gradients flip on/off at the clip bounds (3e-4 wide): compare where the oracle and the
+    # kernel agree on the clip state, i.e. through the total gradient norm-wise at a looser bound
+    g_rt = rt if not gspo else 5e-2
+    assert_close_rel(got["dhidden"], want["dhidden"], g_rt, "dhidden")
+    assert_close_rel(got["dweight"], want["dweight"], g_rt, "dweight")
+    if keep is not None:
+        # masked-out rows were left out of the backward: exact zeros there, and fewer rows projected
+        assert got["rows_projected_bwd"] == int(mask.sum())
+        assert (got["dhidden"][~mask.bool().to(dev)] == 0).all()
+        full = grpo_head_step(d(hidden), d(weight), d(labels), d(old), d(ref), d(adv), d(cu), d(mask),
+                              n_tokens_total=n_tok, use_group_sequence_policy=gspo, pos_clip_ratio=cfg.pos_clip_ratio,
+                              neg_clip_ratio=cfg.neg_clip_ratio, final_clip_ratio=cfg.final_clip_ratio,
+                              kl_coef=cfg.kl_coef, entropy_coef=cfg.entropy_coef, temperature=cfg.temperature,
+                              keep_logits_chunk=keep, cu_seqlens_host=cu.tolist(), skip_masked_rows=False)
+        assert full["rows_projected_bwd"] == T
+        assert_close_rel(got["dhidden"], full["dhidden"], 1e-6 if cfg.dtype == torch.float32 else 1e-2, "skip vs full dh")
+        assert_close_rel(got["dweight"], full["dweight"], 1e-5 if cfg.dtype == torch.float32 else 1e-2, "skip vs full dW")
+
+
+def test_kept_logits_backward_equals_recompute(dev):
+    from chatlearn_amd import ops
+    T, H, V = 700, 256, 5001
+    g = torch.Generator().manual_seed(0)
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    weight = (torch.randn(V, H, generator=g) * 0.05).bfloat16().to(dev)
+    labels = torch.randint(0, V, (T,), generator=g).to(dev)
+    g_lp = torch.randn(T, generator=g).to(dev)
+    g_en = (torch.randn(T, generator=g) * 0.1).to(dev)
+    zbuf = ops.saved_logits_buffer(T, V, torch.bfloat16, dev)
+    lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, 0.8, saved_logits=zbuf)
+    lp2, ent2, _, lse2 = ops.lmhead_forward(hidden, weight, labels, 0.8)
+    assert torch.equal(lp, lp2) and torch.equal(ent, ent2)            # storing logits does not change the statistics
+    z = torch.nn.functional.linear(hidden.float(), weight.float())
+    assert_close_rel(zbuf[:, :V], z, 2 ** -8, "stored logits")        # bf16 rounding of the raw logits
+    assert (zbuf[:, V:] == 0).all()
+    dh1, dw1 = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_en, 0.8)
+    dh2, dw2 = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_en, 0.8, saved_logits=zbuf)
+    assert_close_rel(dh2, dh1, 1e-2, "dhidden kept vs recompute")
+    assert_close_rel(dw2, dw1, 1e-2, "dweight kept vs recompute")

@@ -77,7 +77,8 @@ def test_backward_chunked_equals_unchunked_and_accumulates(dev):
     lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld)
     dh1, dw1 = ops.lmhead_backward(hd, wd, ld, lse, None, gd)
     dh2, dw2 = ops.lmhead_backward(hd, wd, ld, lse, None, gd, chunk_tokens=256)
-    assert torch.equal(dh1, dh2)                      # dhidden rows do not depend on the chunking
+    # dhidden rows do not depend on the chunking beyond the fp32 summation order (split-K differs with M)
+    assert_close_rel(dh2, dh1, 2 ** -7, "chunked dhidden")
     assert_close_rel(dw2, dw1, 1e-5, "chunked dW")   # only the fp32 summation order differs
     base = torch.ones(V, H, device=dev)
     _, dw3 = ops.lmhead_backward(hd, wd, ld, lse, None, gd, dweight=base, accumulate_dweight=True)
