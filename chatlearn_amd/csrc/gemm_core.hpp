@@ -109,65 +109,6 @@ struct GemmTile {
     const int b_frag_off = BM * kRowStride + (wn * WN + (lane & 31)) * kRowStride + (lane >> 5) * 16;
 
     const int nslab = K / kSlabK;
-#if CLGRPO_PREFETCH2
-    // Two register sets: the loads of slab s+2 are issued while slab s is being multiplied and
-    // land in LDS one iteration later, which gives every load about two iterations to arrive.
-    u32x4 ra[2][kPassA], rb[2][kPassB];
-    auto load_set = [&](int set, int slab) {
-      const int koff = slab * kRowBytes;
-#pragma unroll
-      for (int p = 0; p < kPassA; ++p)
-        ra[set][p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, koff, 0);
-#pragma unroll
-      for (int p = 0; p < kPassB; ++p)
-        rb[set][p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, koff, 0);
-    };
-    auto store_set = [&](int set, char* stage) {
-#pragma unroll
-      for (int p = 0; p < kPassA; ++p)
-        *reinterpret_cast<u32x4*>(stage + st_off + p * kRowsPerPass * kRowStride) = ra[set][p];
-#pragma unroll
-      for (int p = 0; p < kPassB; ++p)
-        *reinterpret_cast<u32x4*>(stage + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[set][p];
-    };
-    auto compute = [&](const char* cur) {
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        u32x4 af[MI], bf[NI];
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-          af[mi] = *reinterpret_cast<const u32x4*>(cur + a_frag_off + mi * 32 * kRowStride + kk * 32);
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-          bf[ni] = *reinterpret_cast<const u32x4*>(cur + b_frag_off + ni * 32 * kRowStride + kk * 32);
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-          for (int ni = 0; ni < NI; ++ni) mma_block<T>(acc[mi][ni], af[mi], bf[ni]);
-      }
-    };
-    load_set(0, 0);
-    if (nslab > 1) load_set(1, 1);
-    store_set(0, lds);
-    __syncthreads();
-    // nslab is even for every K this library uses (K is a multiple of 2 slabs) except tiny tests;
-    // the loop handles both parities by unrolling two iterations with fixed register sets.
-    int s = 0;
-    for (; s + 1 < nslab; s += 2) {
-      if (s + 2 < nslab) load_set(0, s + 2);
-      compute(lds);
-      store_set(1, lds + kStageBytes);
-      __syncthreads();
-      if (s + 3 < nslab) load_set(1, s + 3);
-      compute(lds + kStageBytes);
-      if (s + 2 < nslab) store_set(0, lds);
-      __syncthreads();
-    }
-    if (s < nslab) {
-      compute(lds);
-      __syncthreads();
-    }
-#else
     u32x4 ra[kPassA], rb[kPassB];
 
 #pragma unroll
@@ -232,7 +173,6 @@ struct GemmTile {
       }
       __syncthreads();
     }
-#endif
   }
 };
 

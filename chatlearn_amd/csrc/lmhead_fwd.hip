@@ -107,23 +107,54 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
     Tile::run(acc, weight + (int64_t)v0 * p.H, p.H, a_rows, hidden, p.H, b_rows, p.H, lds);
 
     if (STORE_Z) {
-      // Raw logits for the backward: 4 consecutive vocabulary entries of one token per store.
-      // Vocabulary rows past V were read as zero rows of W, so the padding columns hold zeros.
+      // Raw logits for the backward.  Vocabulary rows past V were read as zero rows of W, so the
+      // padding columns hold zeros.
       T* z = static_cast<T*>(p.z_out);
       typedef typename Pack4<T>::type P4;
+      if (sizeof(T) == 2) {
+        // 16-bit logits: turn the tile through LDS (free between two K loops) so that every token
+        // row leaves as whole 16-byte pieces of one contiguous 512-byte run.
+        constexpr int kZRow = kFwdBM * 2 + 16;   // bytes per token row in LDS (padded)
 #pragma unroll
-      for (int ni = 0; ni < NI; ++ni) {
-        if (zrow[ni] >= 0) {
+        for (int ni = 0; ni < NI; ++ni) {
+          char* row = lds + (wn * WN + ni * 32 + (lane & 31)) * kZRow;
 #pragma unroll
           for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const int v_idx = v0 + wm * WM + mi * 32 + 8 * q + 4 * (lane >> 5);
-              if (v_idx < p.ldz)
-                *reinterpret_cast<P4*>(z + (int64_t)zrow[ni] * p.ldz + v_idx) =
-                    Pack4<T>::make(acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
-                                   acc[mi][ni][4 * q + 3]);
-            }
+            for (int q = 0; q < 4; ++q)
+              *reinterpret_cast<P4*>(row + (wm * WM + mi * 32 + 8 * q + 4 * (lane >> 5)) * 2) =
+                  Pack4<T>::make(acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
+                                 acc[mi][ni][4 * q + 3]);
+        }
+        __syncthreads();
+        const int chunk = threadIdx.x & 31;          // 16-byte piece within the 512-byte row
+        const int v_idx = v0 + chunk * 8;
+        if (v_idx < p.ldz) {
+          for (int r = threadIdx.x >> 5; r < kFwdBN; r += Tile::kThreads / 32) {
+            const int tok = t0 + r;
+            int dst = (tok < p.T) ? (p.z_row_map ? p.z_row_map[tok] : tok) : -1;
+            if (dst >= p.z_rows) dst = -1;
+            if (dst >= 0)
+              *reinterpret_cast<u32x4*>(z + (int64_t)dst * p.ldz + v_idx) =
+                  *reinterpret_cast<const u32x4*>(lds + r * kZRow + chunk * 16);
+          }
+        }
+        __syncthreads();   // the next K loop refills the same LDS
+      } else {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+          if (zrow[ni] >= 0) {
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const int v_idx = v0 + wm * WM + mi * 32 + 8 * q + 4 * (lane >> 5);
+                if (v_idx < p.ldz)
+                  *reinterpret_cast<P4*>(z + (int64_t)zrow[ni] * p.ldz + v_idx) =
+                      Pack4<T>::make(acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
+                                     acc[mi][ni][4 * q + 3]);
+              }
+          }
         }
       }
     }
