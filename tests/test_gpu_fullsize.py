@@ -1,0 +1,99 @@
+"""Size-independent properties at the benchmark's full sizes (Qwen3-8B head, 16384 packed
+tokens), where the CPU oracle is too slow to run in full: invariants of the mathematics,
+linearity, determinism, and the oracle on a row sample."""
+import math
+
+import pytest
+import torch
+
+from chatlearn_amd import synthetic
+from oracle import softmax_stats as osm
+from tests.util import assert_close_rel
+
+pytestmark = pytest.mark.gpu
+
+CFG = synthetic.CONFIGS["c2"]
+
+
+@pytest.fixture(scope="module")
+def big(dev):
+    gen = synthetic.generator_for(CFG)
+    samples = synthetic.fill_microbatch(CFG, synthetic.sample_population(CFG, gen))
+    cu, mask = synthetic.packed_layout(samples)
+    T = int(cu[-1])
+    hidden, weight, labels = synthetic.make_head_tensors(CFG, T, gen, device=dev, device_generate=True)
+    return dict(T=T, cu=cu.to(dev), mask=mask.to(dev), hidden=hidden, weight=weight, labels=labels, samples=samples)
+
+
+def test_workload_shape(big):
+    assert big["T"] == CFG.T == 16384 and big["hidden"].shape == (16384, 4096) and big["weight"].shape == (151936, 4096)
+    assert int(big["mask"].sum()) < big["T"]          # prompts are masked out
+
+
+def test_forward_invariants_and_row_sample_vs_oracle(dev, big):
+    from chatlearn_amd import ops
+    lp, ent, mx, lse = ops.lmhead_forward(big["hidden"], big["weight"], big["labels"])
+    assert torch.isfinite(lp).all() and torch.isfinite(ent).all()
+    assert (lp <= 0).all() and (ent > 0).all() and (ent <= math.log(CFG.V) + 1e-3).all()
+    assert (mx <= lse).all() and (lse <= mx + math.log(CFG.V) + 1e-3).all()     # max <= lse <= max + log V
+    lp2, ent2, _, lse2 = ops.lmhead_forward(big["hidden"], big["weight"], big["labels"])
+    assert torch.equal(lp, lp2) and torch.equal(ent, ent2) and torch.equal(lse, lse2)   # run-to-run identical
+    # the oracle on 48 rows spread over the batch (first, last, a tile boundary, random ones)
+    g = torch.Generator().manual_seed(0)
+    rows = torch.cat([torch.tensor([0, 255, 256, 8191, 8192, 16383]), torch.randint(0, big["T"], (42,), generator=g)])
+    h = big["hidden"][rows.to(dev)].cpu()
+    w = big["weight"].cpu()
+    want = osm.fused_head_forward(h, w, big["labels"][rows.to(dev)].cpu(), 1.0, torch.float32)
+    assert_close_rel(lp[rows.to(dev)], want[0], 1e-2, "logprob sample")
+    assert_close_rel(ent[rows.to(dev)], want[1], 1e-2, "entropy sample")
+    # in fact far tighter than the bf16 bound: the fused path keeps fp32 logits
+    assert (lp[rows.to(dev)].cpu() - want[0]).abs().max() < 1e-3
+
+
+def test_backward_invariants_linearity_and_paths_agree(dev, big):
+    from chatlearn_amd import ops
+    T, H, V = big["T"], CFG.H, CFG.V
+    g = torch.Generator(device=dev).manual_seed(1)
+    g1 = torch.randn(T, generator=g, device=dev) * big["mask"]
+    g2 = torch.randn(T, generator=g, device=dev) * big["mask"]
+    zbuf = ops.saved_logits_buffer(T, V, torch.bfloat16, dev)
+    lp, ent, _, lse = ops.lmhead_forward(big["hidden"], big["weight"], big["labels"], saved_logits=zbuf)
+    dh1, dw1 = ops.lmhead_backward(big["hidden"], big["weight"], big["labels"], lse, None, g1, saved_logits=zbuf)
+    # sum_v dz[t,v] = 0  =>  every column of dW sums to ~0 against its own magnitude
+    col = dw1.sum(0)
+    assert col.abs().max() < 2e-3 * dw1.abs().sum(0).max()
+    # rows with zero upstream gradient have exactly zero dhidden
+    assert (dh1[big["mask"] == 0] == 0).all()
+    # the recompute path gives the same gradients (it never saw the bf16-rounded logits)
+    dh1r, dw1r = ops.lmhead_backward(big["hidden"], big["weight"], big["labels"], lse, None, g1)
+    assert_close_rel(dh1, dh1r, 1e-2, "kept-logits vs recompute dhidden")
+    assert_close_rel(dw1, dw1r, 1e-2, "kept-logits vs recompute dW")
+    # linearity in the upstream gradient: bwd(g1) + bwd(g2) = bwd(g1 + g2)
+    dh2, dw2 = ops.lmhead_backward(big["hidden"], big["weight"], big["labels"], lse, None, g2)
+    dh12, dw12 = ops.lmhead_backward(big["hidden"], big["weight"], big["labels"], lse, None, g1 + g2)
+    assert_close_rel(dh1r.float() + dh2.float(), dh12.float(), 1e-2, "linearity dhidden")
+    assert_close_rel(dw1r + dw2, dw12, 1e-2, "linearity dW")
+    # the oracle's closed form on a row sample (dhidden rows are independent of each other)
+    rows = torch.nonzero(big["mask"]).flatten()[::400][:24]
+    h = big["hidden"][rows].cpu()
+    rdh, _ = osm.fused_head_backward_closed_form(h, big["weight"].cpu(), big["labels"][rows].cpu(), g1[rows].cpu(),
+                                                 None, 1.0, torch.float32)
+    assert_close_rel(dh1r[rows], rdh, 1e-2, "dhidden sample vs oracle")
+
+
+def test_head_step_chunkings_agree(dev, big):
+    from chatlearn_amd.fused import grpo_head_step
+    T = big["T"]
+    g = torch.Generator(device=dev).manual_seed(2)
+    lp0 = torch.full((T,), -12.0, device=dev)
+    old = lp0 + torch.randn(T, generator=g, device=dev) * 0.05
+    adv = torch.randn(big["cu"].numel() - 1, generator=g, device=dev)
+    n_tok = float(big["mask"].sum())
+    outs = [grpo_head_step(big["hidden"], big["weight"], big["labels"], old, old, adv, big["cu"], big["mask"],
+                           n_tokens_total=n_tok, kl_coef=1e-3, keep_logits_chunk=k) for k in (8192, 4096)]
+    a, b = outs
+    assert torch.equal(a["logprob"], b["logprob"]) or (a["logprob"] - b["logprob"]).abs().max() < 1e-4
+    assert float(a["total_loss"]) == pytest.approx(float(b["total_loss"]), rel=1e-6)
+    assert_close_rel(a["dhidden"], b["dhidden"], 1e-2, "dhidden 8192 vs 4096 chunks")
+    assert_close_rel(a["dweight"], b["dweight"], 1e-2, "dW 8192 vs 4096 chunks")
+    assert a["rows_projected_bwd"] == b["rows_projected_bwd"] == int(big["mask"].sum())
