@@ -216,4 +216,4 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     return {"logprob": lp_all, "entropy": ent_all, "lse": lse_all, "pg_loss_mean": pg, "kl_loss_mean": kl,
             "entropy_loss_mean": en, "total_loss": total, "num_masked": sums[3],
             "per_token_loss": loss_all, "per_token_kl": kl_all, "dhidden": dh_all, "dweight": dw,
-            "g_logprob": glp_all, "rows_projected_bwd": rows_projected_bwd}
+            "g_logprob": glp_all, "rows_projected_bwd": rows_projected_bwd, "sums": sums}

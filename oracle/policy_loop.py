@@ -1,0 +1,97 @@
+"""Oracle: the FSDP policy trainer's micro-batch loops on one rank, text models.
+
+Test infrastructure only; never imported by the product package.
+
+Reference semantics restated here (sp_size = 1, fsdp_size = 1, no vision inputs):
+  * preprocess_data_list      policy_trainer.py:80-172
+  * train_step loop           policy_trainer.py:203-311   (without optimizer / grad clipping)
+  * forward_step loop         policy_trainer.py:316-365
+
+``model(input_ids, position_ids)`` stands for ``self.model(...).logits``: it returns
+logits [b, s, V].  Everything runs on the CPU with the other oracle modules.
+"""
+import torch
+import torch.nn.functional as F
+
+from . import indexing as oi
+from . import losses as ol
+from . import packing as opk
+from . import softmax_stats as osm
+
+
+def preprocess_data_list(data_list, training, *, packing, max_token_in_seq=None, train_micro_batch_size=1,
+                         generate_micro_batch_size=1):
+    total_resp = torch.tensor(sum(d["response_token_length"] for d in data_list)) / 1   # / sp_size, all-reduce = identity
+    if packing:
+        mbs = opk.split_microbatch(data_list=data_list, max_train_token=max_token_in_seq, packing=True)
+    else:
+        size = train_micro_batch_size if training else generate_micro_batch_size
+        mbs = opk.split_microbatch(data_list=data_list, micro_batch_size=size, packing=False)
+    batches = [opk.batching(mb) for mb in mbs]
+    out = []
+    for b in batches:
+        tokens_ = b["all_tokens"].long()
+        p_len, r_len = b["prompt_token_length"], b["response_token_length"]
+        ori_bs, ori_len = tokens_.size()
+        attn, loss_mask, pos = oi.generate_loss_mask_position_ids(tokens_, p_len, r_len)
+        if "loss_mask" in b:
+            loss_mask = b["loss_mask"]
+        indices = None
+        if packing:
+            tokens_, indices, *_ = oi.unpad_input(tokens_.unsqueeze(-1), attn)
+            tokens_ = tokens_.permute(1, 0)
+            pos, *_ = oi.unpad_input(pos.unsqueeze(-1), attn)
+            pos = pos.permute(1, 0)
+        tokens = tokens_
+        labels = torch.roll(tokens, shifts=-1, dims=1)
+        obj = {"all_tokens": tokens, "position_ids": pos, "labels": labels, "ori_seq_len": ori_len,
+               "indices": indices, "ori_batch_size": ori_bs, "sample_ids": b["id_in_list"],
+               "attention_mask": attn, "pad_size": 0}
+        if training:
+            lm = torch.roll(loss_mask, shifts=-1, dims=1)
+            lm[:, -1] = 0
+            obj.update({"loss_mask": lm, "old_logprobs": b["old_logprobs"], "ref_logprobs": b["ref_logprobs"],
+                        "advantages": b["advantages"]})
+        out.append(obj)
+    return total_resp, out
+
+
+def _repad(x, inputs, packing):
+    if packing:
+        return oi.pad_input(x[0, :x.shape[1] - inputs["pad_size"]].unsqueeze(-1), inputs["indices"],
+                            inputs["ori_batch_size"], inputs["ori_seq_len"]).squeeze(-1)
+    return F.pad(x, (0, inputs["ori_seq_len"] - x.shape[1]), mode="constant", value=0)
+
+
+def train_step(model, data_list, *, packing, module_args, **prep):
+    """Returns (train_stats, per-micro-batch totals); gradients accumulate in the model's parameters."""
+    n_tok, mbs = preprocess_data_list(data_list, True, packing=packing, **prep)
+    pg_l, en_l, kl_l, totals = [], [], [], []
+    for inputs in mbs:
+        logits = model(inputs["all_tokens"], inputs["position_ids"])
+        logprobs = osm.logprobs_from_logits(logits, inputs["labels"])
+        ctx = torch.enable_grad() if module_args["entropy_coef"] > 0 else torch.no_grad()
+        with ctx:
+            entropy = osm.entropy_from_logits_with_chunking(logits)
+        logprobs, entropy = _repad(logprobs, inputs, packing), _repad(entropy, inputs, packing)
+        total, parts = ol.fsdp_policy_loss(
+            logprobs, entropy, inputs["old_logprobs"], inputs["ref_logprobs"], inputs["advantages"],
+            inputs["loss_mask"], n_tok, entropy_coef=module_args["entropy_coef"], kl_coef=module_args["kl_coef"],
+            pos_clip_ratio=module_args.get("pos_clip_ratio", 0.2), neg_clip_ratio=module_args.get("neg_clip_ratio", 0.2),
+            diff_clip_ratio=module_args.get("diff_clip_ratio", 10), final_clip_ratio=module_args.get("final_clip_ratio", 3))
+        total.backward()
+        totals.append(total.detach())
+        pg_l.append(parts["pg_loss"]); en_l.append(parts["entropy_loss"]); kl_l.append(parts["kl_loss"])
+    return ol.fsdp_train_metrics(pg_l, en_l, kl_l, n_tok), totals
+
+
+def forward_step(model, data, *, packing, trainable, **prep):
+    _, mbs = preprocess_data_list(data, False, packing=packing, **prep)
+    tag = "old_logprobs" if trainable else "ref_logprobs"
+    for inputs in mbs:
+        with torch.no_grad():
+            logits = model(inputs["all_tokens"], inputs["position_ids"])
+            logprobs = _repad(osm.logprobs_from_logits(logits, inputs["labels"]), inputs, packing)
+        for sid, lp in zip(inputs["sample_ids"], oi.split_and_unpadding(logprobs, inputs["attention_mask"])):
+            data[sid].update({tag: lp})
+    return data
