@@ -149,6 +149,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-unfused", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 1 GiB device copies (a kernel of known HBM traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--no-skip-masked", action="store_true",
                     help="run the backward on every row, also those whose loss mask is zero")
     ap.add_argument("--keep-logits-chunk", type=int, default=8192,
@@ -208,6 +211,14 @@ def main():
         if record:
             marks.append(cur)
         return out
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     out_last = None
     for _ in range(args.warmup):

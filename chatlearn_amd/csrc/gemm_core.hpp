@@ -6,7 +6,9 @@
 // elements).  A slab of A (BM rows) and of B (BN rows) is staged in LDS with a
 // padded row stride of 144 bytes, which keeps the 16-byte fragment reads of 16
 // consecutive rows on distinct banks.  Two LDS stages: while the matrix cores
-// work on stage s, the next slab travels HBM/L2 -> registers -> stage s^1.
+// work on stage s, the next slab travels HBM/L2 -> registers -> stage s^1; the
+// fragment reads, global loads and LDS stores are spread between the matrix
+// instructions and the workgroup barrier sits before the last K-step of a slab.
 //
 // Accumulator layout (v_mfma_f32_32x32x*): for the 32x32 block (mi, ni) of a
 // wave, lane l, register r hold
@@ -109,70 +111,103 @@ struct GemmTile {
     const int b_frag_off = BM * kRowStride + (wn * WN + (lane & 31)) * kRowStride + (lane >> 5) * 16;
 
     const int nslab = K / kSlabK;
+    // Branch-free slab loop.  Per slab: four K-steps of MI*NI matrix instructions; the fragment
+    // reads of the next K-step, the global loads of the next slab and its LDS stores are spread
+    // between the matrix instructions, and the workgroup barrier sits before the last K-step, so
+    // that step's matrix instructions cover the first fragment reads of the next slab.
     u32x4 ra[kPassA], rb[kPassB];
+    u32x4 af[2][MI], bf[2][NI];
+    const int last = nslab - 1;
+    auto load_slab = [&](int slab) {
+      const int koff = (slab < last ? slab : last) * kRowBytes;   // clamped: always in bounds
+#pragma unroll
+      for (int p = 0; p < kPassA; ++p)
+        ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, koff, 0);
+#pragma unroll
+      for (int p = 0; p < kPassB; ++p)
+        rb[p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, koff, 0);
+    };
+    auto store_slab = [&](char* stage) {
+#pragma unroll
+      for (int p = 0; p < kPassA; ++p)
+        *reinterpret_cast<u32x4*>(stage + st_off + p * kRowsPerPass * kRowStride) = ra[p];
+#pragma unroll
+      for (int p = 0; p < kPassB; ++p)
+        *reinterpret_cast<u32x4*>(stage + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[p];
+    };
+    auto read_frags = [&](int set, const char* stage, int kk) {
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+        af[set][mi] = *reinterpret_cast<const u32x4*>(stage + a_frag_off + mi * 32 * kRowStride + kk * 32);
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+        bf[set][ni] = *reinterpret_cast<const u32x4*>(stage + b_frag_off + ni * 32 * kRowStride + kk * 32);
+    };
+    auto mma = [&](int set) {
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) mma_block<T>(acc[mi][ni], af[set][mi], bf[set][ni]);
+    };
 
-#pragma unroll
-    for (int p = 0; p < kPassA; ++p) ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, 0, 0);
-#pragma unroll
-    for (int p = 0; p < kPassB; ++p) rb[p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, 0, 0);
-#pragma unroll
-    for (int p = 0; p < kPassA; ++p)
-      *reinterpret_cast<u32x4*>(lds + st_off + p * kRowsPerPass * kRowStride) = ra[p];
-#pragma unroll
-    for (int p = 0; p < kPassB; ++p)
-      *reinterpret_cast<u32x4*>(lds + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[p];
+    load_slab(0);
+    store_slab(lds);
+    load_slab(1);
     __syncthreads();
-
+    read_frags(0, lds, 0);
     for (int s = 0; s < nslab; ++s) {
       char* cur = lds + (s & 1) * kStageBytes;
       char* nxt = lds + ((s & 1) ^ 1) * kStageBytes;
-      const bool more = (s + 1) < nslab;
-      if (more) {
-        const int koff = (s + 1) * kRowBytes;
+      // K-step 0: fragments of step 1 come in between the matrix instructions
+      read_frags(1, cur, 1);
+      mma(0);
 #pragma unroll
-        for (int p = 0; p < kPassA; ++p)
-          ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, koff, 0);
-#pragma unroll
-        for (int p = 0; p < kPassB; ++p)
-          rb[p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, koff, 0);
+      for (int i = 0; i < MI + NI; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-      // Fragments of K-step kk+1 are fetched from LDS before the matrix
-      // instructions of step kk are issued, so the LDS latency hides behind them.
-      u32x4 af[2][MI], bf[2][NI];
+      __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - (MI + NI), 0);
+      // K-step 1
+      read_frags(0, cur, 2);
+      mma(1);
 #pragma unroll
-      for (int mi = 0; mi < MI; ++mi)
-        af[0][mi] = *reinterpret_cast<const u32x4*>(cur + a_frag_off + mi * 32 * kRowStride);
-#pragma unroll
-      for (int ni = 0; ni < NI; ++ni)
-        bf[0][ni] = *reinterpret_cast<const u32x4*>(cur + b_frag_off + ni * 32 * kRowStride);
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        if (kk < 3) {
-#pragma unroll
-          for (int mi = 0; mi < MI; ++mi)
-            af[(kk + 1) & 1][mi] =
-                *reinterpret_cast<const u32x4*>(cur + a_frag_off + mi * 32 * kRowStride + (kk + 1) * 32);
-#pragma unroll
-          for (int ni = 0; ni < NI; ++ni)
-            bf[(kk + 1) & 1][ni] =
-                *reinterpret_cast<const u32x4*>(cur + b_frag_off + ni * 32 * kRowStride + (kk + 1) * 32);
-        }
-        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of this step's matrix ops
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-          for (int ni = 0; ni < NI; ++ni) mma_block<T>(acc[mi][ni], af[kk & 1][mi], bf[kk & 1][ni]);
+      for (int i = 0; i < MI + NI; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-      if (more) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - (MI + NI), 0);
+      // K-step 2: fragments of step 3 and the LDS stores of the next slab
+      read_frags(1, cur, 3);
+      store_slab(nxt);
+      mma(0);
 #pragma unroll
-        for (int p = 0; p < kPassA; ++p)
-          *reinterpret_cast<u32x4*>(nxt + st_off + p * kRowsPerPass * kRowStride) = ra[p];
-#pragma unroll
-        for (int p = 0; p < kPassB; ++p)
-          *reinterpret_cast<u32x4*>(nxt + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[p];
+      for (int i = 0; i < MI + NI; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
+#pragma unroll
+      for (int i = 0; i < MI * NI - (MI + NI); ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x200, (kPassA + kPassB + 1) / 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x200, kPassA + kPassB, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // everyone has the last fragments of `cur` in registers and has written its part of `nxt`
       __syncthreads();
+      // K-step 3 covers the first fragment reads of the next slab and the next global loads
+      read_frags(0, nxt, 0);
+      load_slab(s + 2);
+      mma(1);
+#pragma unroll
+      for (int i = 0; i < MI + NI; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, (kPassA + kPassB + MI + NI - 1) / (MI + NI), 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - (MI + NI), 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    __syncthreads();   // the caller may reuse LDS; every wave is past its last fragment read
   }
 };
 
