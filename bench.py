@@ -28,6 +28,12 @@ from chatlearn_amd._lib import LOSS_GRPO, LOSS_GSPO  # noqa: E402
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3
 
+# HBM-side bytes (L2 <-> fabric, read + written) of ONE forward launch, from two rocprofv3 --pmc runs
+# (FETCH_SIZE scaled by 2.00, WRITE_SIZE by 1.00 after a plain 1 GiB copy calibration; the summary is
+# kept with the other profiles).  Key: (config, tokens per launch, chunk logits kept).  Other
+# workloads have not been measured and report null.
+MEASURED_FWD_TRAFFIC_BYTES = {("c2", 8192, True): 30.35e9}
+
 
 def build_workload(cfg, device):
     gen = synthetic.generator_for(cfg)
@@ -140,6 +146,28 @@ def unfused_gpu(cfg, hidden, weight, labels, old, ref, adv, cu, mask, n_tok, ste
     return (time.perf_counter() - t0) / steps
 
 
+def library_gemms(hidden, weight, reps=5):
+    """Plain library GEMMs (no softmax, logits materialised) at the head shape: the practical
+    ceiling of this GPU's matrix cores under sustained load, for context next to the fused kernels."""
+    T, H = hidden.shape
+    V = weight.shape[0]
+    flops = 2.0 * T * H * V
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return flops / (e0.elapsed_time(e1) / reps * 1e-3) / 1e12
+    z = torch.nn.functional.linear(hidden, weight)
+    return {"unit": "TFLOP/s", "logits = hidden @ W^T": timed(lambda: torch.nn.functional.linear(hidden, weight)),
+            "dhidden = dlogits @ W": timed(lambda: z @ weight), "dW = dlogits^T @ hidden": timed(lambda: z.t() @ hidden)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -149,6 +177,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-unfused", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256)
+    ap.add_argument("--gemm-reference", action="store_true",
+                    help="also time the vendor library's plain GEMMs (torch.matmul) at this head shape, for context")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (a kernel of known HBM traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -265,7 +295,8 @@ def main():
                    "token_chunks": [hi - lo for lo, hi in chunks], "logits_kept_per_chunk": bool(keep),
                    "T_projected_forward": T, "T_projected_backward": rows_bwd},
         "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tflops, "peak": peak,
-                     "unit": "TFLOP/s", "frac": fwd_tflops / peak, "traffic": None,
+                     "unit": "TFLOP/s", "frac": fwd_tflops / peak,
+                     "traffic": MEASURED_FWD_TRAFFIC_BYTES.get((cfg.name, max(hi - lo for lo, hi in chunks), bool(keep))),
                      "algorithmic_flops_per_launch": 2.0 * thv / n_fwd_launch,
                      "avg_launch_ms": fwd_ms / n_fwd_launch, "launches_per_step": n_fwd_launch},
         "step_mfma_frac": step_flops / dt / 1e12 / peak,
@@ -278,6 +309,8 @@ def main():
                                         "speedup_fused": u_dt / dt}
         except Exception as e:  # the unfused path can run out of memory on large configs
             out["unfused_torch_gpu"] = {"error": str(e)[:200]}
+    if args.gemm_reference:
+        out["library_gemm_reference"] = library_gemms(hidden, weight)
     if not args.no_cpu_baseline:
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
         tps, reps = cpu_baseline(cfg, args.cpu_rows, threads)
