@@ -112,28 +112,31 @@ struct GemmTile {
 
     const int nslab = K / kSlabK;
     // Branch-free slab loop.  Per slab: four K-steps of MI*NI matrix instructions; the fragment
-    // reads of the next K-step, the global loads of the next slab and its LDS stores are spread
-    // between the matrix instructions, and the workgroup barrier sits before the last K-step, so
-    // that step's matrix instructions cover the first fragment reads of the next slab.
-    u32x4 ra[kPassA], rb[kPassB];
+    // reads of the next K-step, the global loads of a later slab and the LDS stores of the next
+    // slab are spread between the matrix instructions, and the workgroup barrier sits before the
+    // last K-step, so that step's matrix instructions cover the first fragment reads of the next
+    // slab.  kSets register sets stage the global loads; with two sets a slab's loads would be
+    // issued one and a half slabs before they are stored to LDS (kept for a lower-occupancy tile).
+    constexpr int kSets = 1;   // two sets need more registers than eight waves per workgroup leave
+    u32x4 ra[kSets][kPassA], rb[kSets][kPassB];
     u32x4 af[2][MI], bf[2][NI];
     const int last = nslab - 1;
-    auto load_slab = [&](int slab) {
+    auto load_slab = [&](int set, int slab) {
       const int koff = (slab < last ? slab : last) * kRowBytes;   // clamped: always in bounds
 #pragma unroll
       for (int p = 0; p < kPassA; ++p)
-        ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, koff, 0);
+        ra[set][p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, koff, 0);
 #pragma unroll
       for (int p = 0; p < kPassB; ++p)
-        rb[p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, koff, 0);
+        rb[set][p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, koff, 0);
     };
-    auto store_slab = [&](char* stage) {
+    auto store_slab = [&](int set, char* stage) {
 #pragma unroll
       for (int p = 0; p < kPassA; ++p)
-        *reinterpret_cast<u32x4*>(stage + st_off + p * kRowsPerPass * kRowStride) = ra[p];
+        *reinterpret_cast<u32x4*>(stage + st_off + p * kRowsPerPass * kRowStride) = ra[set][p];
 #pragma unroll
       for (int p = 0; p < kPassB; ++p)
-        *reinterpret_cast<u32x4*>(stage + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[p];
+        *reinterpret_cast<u32x4*>(stage + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[set][p];
     };
     auto read_frags = [&](int set, const char* stage, int kk) {
 #pragma unroll
@@ -149,63 +152,90 @@ struct GemmTile {
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) mma_block<T>(acc[mi][ni], af[set][mi], bf[set][ni]);
     };
-
-    load_slab(0);
-    store_slab(lds);
-    load_slab(1);
-    __syncthreads();
-    read_frags(0, lds, 0);
-    for (int s = 0; s < nslab; ++s) {
-      char* cur = lds + (s & 1) * kStageBytes;
-      char* nxt = lds + ((s & 1) ^ 1) * kStageBytes;
-      // K-step 0: fragments of step 1 come in between the matrix instructions
-      read_frags(1, cur, 1);
-      mma(0);
+    constexpr int kFragReads = MI + NI;
+    constexpr int kMma = MI * NI;
+    constexpr int kLoads = kPassA + kPassB;
+    constexpr int kFree = kMma - kFragReads > 0 ? kMma - kFragReads : 1;   // matrix ops left after the fragment reads
+    // one K-step: `kFragReads` matrix ops each followed by one LDS read, then the rest
+    auto pace_reads = [&]() {
 #pragma unroll
-      for (int i = 0; i < MI + NI; ++i) {
+      for (int i = 0; i < kFragReads; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - (MI + NI), 0);
+    };
+    // one slab; `st` = register set holding slab s+1, `ld` = set that receives a later slab
+    auto slab_body = [&](int s, int st, int ld, char* cur, char* nxt) {
+      // K-step 0 (two sets: the loads of slab s+2 ride along here)
+      read_frags(1, cur, 1);
+      if (kSets == 2) load_slab(ld, s + 2);
+      mma(0);
+      if (kSets == 2) {
+#pragma unroll
+        for (int i = 0; i < kFragReads; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, (kLoads + kFragReads - 1) / kFragReads, 0);
+        }
+      } else {
+        pace_reads();
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kMma - kFragReads, 0);
       // K-step 1
       read_frags(0, cur, 2);
       mma(1);
-#pragma unroll
-      for (int i = 0; i < MI + NI; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - (MI + NI), 0);
+      pace_reads();
+      __builtin_amdgcn_sched_group_barrier(0x008, kMma - kFragReads, 0);
       // K-step 2: fragments of step 3 and the LDS stores of the next slab
       read_frags(1, cur, 3);
-      store_slab(nxt);
+      store_slab(st, nxt);
       mma(0);
+      pace_reads();
 #pragma unroll
-      for (int i = 0; i < MI + NI; ++i) {
+      for (int i = 0; i < kFree; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x200, (kLoads + kFree - 1) / kFree, 0);
       }
-#pragma unroll
-      for (int i = 0; i < MI * NI - (MI + NI); ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x200, (kPassA + kPassB + 1) / 2, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x200, kPassA + kPassB, 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, kLoads, 0);
       __builtin_amdgcn_sched_barrier(0);
       // everyone has the last fragments of `cur` in registers and has written its part of `nxt`
       __syncthreads();
-      // K-step 3 covers the first fragment reads of the next slab and the next global loads
+      // K-step 3 covers the first fragment reads of the next slab (one set: and the next global loads)
       read_frags(0, nxt, 0);
-      load_slab(s + 2);
+      if (kSets == 1) load_slab(ld, s + 2);
       mma(1);
+      if (kSets == 1) {
 #pragma unroll
-      for (int i = 0; i < MI + NI; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x020, (kPassA + kPassB + MI + NI - 1) / (MI + NI), 0);
+        for (int i = 0; i < kFragReads; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, (kLoads + kFragReads - 1) / kFragReads, 0);
+        }
+      } else {
+        pace_reads();
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - (MI + NI), 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, kMma - kFragReads, 0);
       __builtin_amdgcn_sched_barrier(0);
+    };
+
+    load_slab(0, 0);
+    if (kSets == 2) {
+      load_slab(1, 1);
+      store_slab(0, lds);
+      __syncthreads();
+      read_frags(0, lds, 0);
+      for (int s = 0; s < nslab; s += 2) {
+        slab_body(s, 1, 0, lds, lds + kStageBytes);
+        if (s + 1 >= nslab) break;
+        slab_body(s + 1, 0, 1, lds + kStageBytes, lds);
+      }
+    } else {
+      store_slab(0, lds);
+      load_slab(0, 1);
+      __syncthreads();
+      read_frags(0, lds, 0);
+      for (int s = 0; s < nslab; ++s)
+        slab_body(s, 0, 0, lds + (s & 1) * kStageBytes, lds + ((s & 1) ^ 1) * kStageBytes);
     }
     __syncthreads();   // the caller may reuse LDS; every wave is past its last fragment read
   }
