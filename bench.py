@@ -182,6 +182,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (a kernel of known HBM traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--skip-masked-forward", action="store_true",
+                    help="also leave rows whose loss mask is zero out of the forward (their per-token outputs become zero)")
     ap.add_argument("--no-skip-masked", action="store_true",
                     help="run the backward on every row, also those whose loss mask is zero")
     ap.add_argument("--keep-logits-chunk", type=int, default=8192,
@@ -236,7 +238,8 @@ def main():
                              final_clip_ratio=cfg.final_clip_ratio, kl_coef=cfg.kl_coef,
                              entropy_coef=cfg.entropy_coef, temperature=cfg.temperature, dweight=dweight,
                              accumulate_dweight=False, keep_logits_chunk=keep, cu_seqlens_host=cu_host,
-                             skip_masked_rows=not args.no_skip_masked, stage_hook=hook if record else None,
+                             skip_masked_rows=not args.no_skip_masked, skip_masked_forward=args.skip_masked_forward,
+                             stage_hook=hook if record else None,
                              check_flags=False)
         if record:
             marks.append(cur)
@@ -270,6 +273,7 @@ def main():
     fwd_ms, loss_ms, bwd_ms = stage_ms("forward"), stage_ms("loss"), stage_ms("backward")
     n_fwd_launch = len(chunks) if train else 1
     rows_bwd = out_last["rows_projected_bwd"] if train else 0
+    rows_fwd = out_last["rows_projected_fwd"] if train else T
 
     thv = float(T) * cfg.H * cfg.V
     peak = PEAK_BF16_TFLOPS if cfg.dtype == torch.bfloat16 else PEAK_F32_TFLOPS
@@ -293,7 +297,7 @@ def main():
                                f"{' fwd+bwd (dhidden ' + str(cfg.dtype).split('.')[-1] + ', dW fp32)' if train else ''}",
                    "temperature": cfg.temperature, "kl_coef": cfg.kl_coef, "entropy_coef": cfg.entropy_coef,
                    "token_chunks": [hi - lo for lo, hi in chunks], "logits_kept_per_chunk": bool(keep),
-                   "T_projected_forward": T, "T_projected_backward": rows_bwd},
+                   "T_projected_forward": rows_fwd, "T_projected_backward": rows_bwd},
         "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tflops, "peak": peak,
                      "unit": "TFLOP/s", "frac": fwd_tflops / peak,
                      "traffic": MEASURED_FWD_TRAFFIC_BYTES.get((cfg.name, max(hi - lo for lo, hi in chunks), bool(keep))),

@@ -130,7 +130,9 @@ class PolicyStep:
                 diff_clip_ratio=args["diff_clip_ratio"], final_clip_ratio=args["final_clip_ratio"],
                 kl_coef=args["kl_coef"], entropy_coef=args["entropy_coef"], temperature=self.temperature, dweight=dw,
                 accumulate_dweight=accumulate, need_dhidden=flat.requires_grad,
-                keep_logits_chunk=self.keep_logits_chunk)
+                keep_logits_chunk=self.keep_logits_chunk,
+                # only masked sums leave this method, so rows outside the loss mask need no forward either
+                skip_masked_forward=True)
             dw, accumulate = out["dweight"], True
             if flat.requires_grad:
                 hidden.backward(out["dhidden"].reshape(hidden.shape))

@@ -99,7 +99,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                    kl_coef=0.0, entropy_coef=0.0, temperature=1.0, dweight: Optional[torch.Tensor] = None,
                    accumulate_dweight=False, need_dhidden=True, check_flags=True,
                    keep_logits_chunk: Optional[int] = 8192, cu_seqlens_host=None, skip_masked_rows=True,
-                   stage_hook=None):
+                   skip_masked_forward=False, stage_hook=None):
     """Forward + loss + backward of the head for one packed micro-batch, no autograd graph.
 
     Mirrors policy_trainer.py:216-286 on packed rows: returns a dict with the
@@ -117,6 +117,12 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     ``skip_masked_rows`` (only with kept logits and a loss mask): rows whose mask is zero have an
     exactly zero upstream gradient, so the backward runs on the compacted set of the other rows
     (their dhidden rows are zero); ``rows_projected_bwd`` in the result counts the rows it ran on.
+
+    ``skip_masked_forward`` (off by default, needs ``skip_masked_rows``): also leave those rows out of
+    the forward.  The loss, its sums and every gradient are unchanged (masked rows enter none of
+    them), but the returned per-token ``logprob`` / ``entropy`` / ``lse`` are zero at masked rows
+    instead of the values the reference computes and then ignores; ``rows_projected_fwd`` counts
+    the rows the forward ran on.
 
     ``stage_hook(name)`` is called on the host at "forward", "loss", "backward", "end" boundaries
     of every chunk (a benchmark records stream events there).
@@ -143,6 +149,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     dw = dweight
     acc_dw = accumulate_dweight
     rows_projected_bwd = 0
+    rows_projected_fwd = 0
     wt = ops.weight_t_buffer(weight) if (need_dhidden and len(chunks) > 1) else None
     wt_ready = False
     kl_c = kl_coef if kl_coef > 0 else 0.0
@@ -158,8 +165,19 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
             row_map = torch.full((n,), -1, dtype=torch.int32, device=hidden.device)
             row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
         hook("forward")
-        lp, ent, _, lse = ops.lmhead_forward(hidden[sl], weight, labels[sl], temperature, need_entropy=True,
-                                             saved_logits=zbuf, saved_row_map=row_map)
+        h_c = lab_c = None
+        if live is not None and skip_masked_forward and live.numel() > 0:
+            # forward on the compact set of unmasked rows; results scattered back, zeros elsewhere
+            h_c, lab_c = ops.gather_rows(hidden[sl], live), ops.gather_rows(labels[sl].reshape(n, 1), live).reshape(-1)
+            lp_c, ent_c, _, lse_c = ops.lmhead_forward(h_c, weight, lab_c, temperature, need_entropy=True,
+                                                       saved_logits=zbuf)
+            spread = lambda x: ops.scatter_rows(x.reshape(-1, 1), live, n).reshape(-1)
+            lp, ent, lse = spread(lp_c), spread(ent_c), spread(lse_c)
+            rows_projected_fwd += int(live.numel())
+        else:
+            lp, ent, _, lse = ops.lmhead_forward(hidden[sl], weight, labels[sl], temperature, need_entropy=True,
+                                                 saved_logits=zbuf, saved_row_map=row_map)
+            rows_projected_fwd += n
         hook("loss")
         res = ops.policy_loss(
             lp, old_logprob[sl], advantages, mode=mode, cu_seqlens=cu_seqlens,
@@ -182,8 +200,10 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                     else dw.zero_()
         else:
             pick = lambda x: None if x is None else ops.gather_rows(x.reshape(n, -1), live).reshape(-1)
+            if h_c is None:
+                h_c, lab_c = ops.gather_rows(hidden[sl], live), pick(labels[sl])
             dh_c, dw = ops.lmhead_backward(
-                ops.gather_rows(hidden[sl], live), weight, pick(labels[sl]), pick(lse), pick(ent),
+                h_c, weight, lab_c, pick(lse), pick(ent),
                 pick(res.g_logprob), pick(res.g_entropy), temperature, need_dhidden=need_dhidden,
                 need_dweight=True, dweight=dw, accumulate_dweight=acc_dw, saved_logits=zbuf, weight_t=wt,
                 weight_t_ready=wt_ready)
@@ -216,4 +236,5 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     return {"logprob": lp_all, "entropy": ent_all, "lse": lse_all, "pg_loss_mean": pg, "kl_loss_mean": kl,
             "entropy_loss_mean": en, "total_loss": total, "num_masked": sums[3],
             "per_token_loss": loss_all, "per_token_kl": kl_all, "dhidden": dh_all, "dweight": dw,
-            "g_logprob": glp_all, "rows_projected_bwd": rows_projected_bwd, "sums": sums}
+            "g_logprob": glp_all, "rows_projected_bwd": rows_projected_bwd,
+            "rows_projected_fwd": rows_projected_fwd, "sums": sums}

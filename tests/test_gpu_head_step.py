@@ -71,7 +71,20 @@ def test_head_step_matches_oracle(dev, name, kw, keep):
                               neg_clip_ratio=cfg.neg_clip_ratio, final_clip_ratio=cfg.final_clip_ratio,
                               kl_coef=cfg.kl_coef, entropy_coef=cfg.entropy_coef, temperature=cfg.temperature,
                               keep_logits_chunk=keep, cu_seqlens_host=cu.tolist(), skip_masked_rows=False)
-        assert full["rows_projected_bwd"] == T
+        assert full["rows_projected_bwd"] == T and full["rows_projected_fwd"] == T
+        lean = grpo_head_step(d(hidden), d(weight), d(labels), d(old), d(ref), d(adv), d(cu), d(mask),
+                              n_tokens_total=n_tok, use_group_sequence_policy=gspo, pos_clip_ratio=cfg.pos_clip_ratio,
+                              neg_clip_ratio=cfg.neg_clip_ratio, final_clip_ratio=cfg.final_clip_ratio,
+                              kl_coef=cfg.kl_coef, entropy_coef=cfg.entropy_coef, temperature=cfg.temperature,
+                              keep_logits_chunk=keep, cu_seqlens_host=cu.tolist(), skip_masked_forward=True)
+        # forward on unmasked rows only: same loss and gradients, zeros at masked rows of the per-token outputs
+        assert lean["rows_projected_fwd"] == int(mask.sum())
+        assert float(lean["total_loss"]) == pytest.approx(float(got["total_loss"]), rel=1e-6)
+        keep_rows = mask.bool().to(dev)
+        assert (lean["logprob"][~keep_rows] == 0).all()
+        assert (lean["logprob"][keep_rows] - got["logprob"][keep_rows]).abs().max() < 1e-4
+        assert_close_rel(lean["dhidden"], got["dhidden"], 1e-6 if cfg.dtype == torch.float32 else 1e-2, "lean dh")
+        assert_close_rel(lean["dweight"], got["dweight"], 1e-5 if cfg.dtype == torch.float32 else 1e-2, "lean dW")
         assert_close_rel(got["dhidden"], full["dhidden"], 1e-6 if cfg.dtype == torch.float32 else 1e-2, "skip vs full dh")
         assert_close_rel(got["dweight"], full["dweight"], 1e-5 if cfg.dtype == torch.float32 else 1e-2, "skip vs full dW")
 
