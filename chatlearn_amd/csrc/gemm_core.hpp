@@ -3,12 +3,15 @@
 //
 // One workgroup of WAVES_M x WAVES_N wavefronts (64 lanes each) owns a BM x BN
 // tile.  K is walked in slabs of 128 bytes per row (64 bf16 or 32 fp32
-// elements).  A slab of A (BM rows) and of B (BN rows) is staged in LDS with a
-// padded row stride of 144 bytes, which keeps the 16-byte fragment reads of 16
-// consecutive rows on distinct banks.  Two LDS stages: while the matrix cores
-// work on stage s, the next slab travels HBM/L2 -> registers -> stage s^1; the
-// fragment reads, global loads and LDS stores are spread between the matrix
-// instructions and the workgroup barrier sits before the last K-step of a slab.
+// elements).  A slab of A (BM rows) and of B (BN rows) travels HBM/L2 -> LDS
+// directly (buffer loads with an LDS destination; no registers, no LDS store
+// instructions).  Such a load fills LDS in lane order, so rows are 128 bytes
+// apart with no padding; bank conflicts are avoided by an XOR swizzle of the
+// 16-byte K-chunks within a row, applied on the global side of the load and
+// undone by the fragment reads.  Two LDS stages: while the matrix cores work on
+// stage s, the next slab lands in stage s^1; one workgroup barrier per slab,
+// placed before the last K-step so that step's matrix instructions cover the
+// first fragment reads of the next slab.
 //
 // Accumulator layout (v_mfma_f32_32x32x*): for the 32x32 block (mi, ni) of a
 // wave, lane l, register r hold
@@ -29,7 +32,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kRowBytes = 128;    // K-slab bytes per tile row
-constexpr int kRowStride = 144;   // LDS row stride in bytes (128 + 16 pad)
 constexpr int kChunksPerRow = 8;  // 16-byte chunks per slab row
 
 template <typename T> struct Elem;
@@ -71,7 +73,7 @@ struct GemmTile {
   static constexpr int MI = WM / 32, NI = WN / 32;
   static constexpr int kRowsPerPass = kThreads / kChunksPerRow;
   static constexpr int kPassA = BM / kRowsPerPass, kPassB = BN / kRowsPerPass;
-  static constexpr int kStageBytes = (BM + BN) * kRowStride;
+  static constexpr int kStageBytes = (BM + BN) * kRowBytes;
   static constexpr int kLdsBytes = 2 * kStageBytes;
   static constexpr int kSlabK = Elem<T>::kSlabK;
   static_assert(BM % kRowsPerPass == 0 && BN % kRowsPerPass == 0, "tile rows vs threads");
@@ -101,50 +103,51 @@ struct GemmTile {
         const_cast<T*>(a_base), 0, a_rows * lda_b, 0x00020000);
     const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<T*>(b_base), 0, b_rows * ldb_b, 0x00020000);
-    const int a_voff = ld_row * lda_b + ld_chunk * 16;
-    const int b_voff = ld_row * ldb_b + ld_chunk * 16;
+    // A wave's load instruction fills 1 KB of LDS in lane order: 8 rows x 8 chunks of 16 bytes.
+    // The lane that lands on (row, slot) fetches K-chunk slot ^ swz(row), so a fragment read of
+    // K-chunk q goes to slot q ^ swz(row).
+    const int ld_swz = (ld_row & 7) ^ ((ld_row >> 3) & 1);
+    const int a_voff = ld_row * lda_b + ((ld_chunk ^ ld_swz) * 16);
+    const int b_voff = ld_row * ldb_b + ((ld_chunk ^ ld_swz) * 16);
     const int a_pass = kRowsPerPass * lda_b;
     const int b_pass = kRowsPerPass * ldb_b;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int dma_off = wave_u * 8 * kRowBytes;   // LDS offset of this wave's 8 rows within a pass
 
-    const int st_off = ld_row * kRowStride + ld_chunk * 16;
-    const int a_frag_off = (wm * WM + (lane & 31)) * kRowStride + (lane >> 5) * 16;
-    const int b_frag_off = BM * kRowStride + (wn * WN + (lane & 31)) * kRowStride + (lane >> 5) * 16;
+    const int fr_swz = (lane & 7) ^ ((lane >> 3) & 1);
+    int xk[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) xk[kk] = ((kk * 2 + (lane >> 5)) ^ fr_swz) * 16;
+    const int a_frag_off = (wm * WM + (lane & 31)) * kRowBytes;
+    const int b_frag_off = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
 
+    typedef __attribute__((address_space(3))) char lds_char;
     const int nslab = K / kSlabK;
-    // Branch-free slab loop.  Per slab: four K-steps of MI*NI matrix instructions; the fragment
-    // reads of the next K-step, the global loads of a later slab and the LDS stores of the next
-    // slab are spread between the matrix instructions, and the workgroup barrier sits before the
-    // last K-step, so that step's matrix instructions cover the first fragment reads of the next
-    // slab.  kSets register sets stage the global loads; with two sets a slab's loads would be
-    // issued one and a half slabs before they are stored to LDS (kept for a lower-occupancy tile).
-    constexpr int kSets = 1;   // two sets need more registers than eight waves per workgroup leave
-    u32x4 ra[kSets][kPassA], rb[kSets][kPassB];
     u32x4 af[2][MI], bf[2][NI];
     const int last = nslab - 1;
-    auto load_slab = [&](int set, int slab) {
+    // global -> LDS without passing registers; completion is awaited before the next barrier
+    auto dma_slab = [&](char* stage, int slab) {
       const int koff = (slab < last ? slab : last) * kRowBytes;   // clamped: always in bounds
+      lds_char* dst = (lds_char*)(stage) + dma_off;
 #pragma unroll
       for (int p = 0; p < kPassA; ++p)
-        ra[set][p] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + p * a_pass, koff, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, dst + p * kRowsPerPass * kRowBytes, 16,
+                                                 a_voff + p * a_pass, koff, 0, 0);
 #pragma unroll
       for (int p = 0; p < kPassB; ++p)
-        rb[set][p] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff + p * b_pass, koff, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, dst + (BM + p * kRowsPerPass) * kRowBytes, 16,
+                                                 b_voff + p * b_pass, koff, 0, 0);
     };
-    auto store_slab = [&](int set, char* stage) {
-#pragma unroll
-      for (int p = 0; p < kPassA; ++p)
-        *reinterpret_cast<u32x4*>(stage + st_off + p * kRowsPerPass * kRowStride) = ra[set][p];
-#pragma unroll
-      for (int p = 0; p < kPassB; ++p)
-        *reinterpret_cast<u32x4*>(stage + BM * kRowStride + st_off + p * kRowsPerPass * kRowStride) = rb[set][p];
-    };
+    // A workgroup barrier does not wait for loads whose destination is LDS: wait for this wave's
+    // outstanding ones explicitly (s_waitcnt vmcnt(0), the other counters left alone).
+    auto wait_loads = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
     auto read_frags = [&](int set, const char* stage, int kk) {
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi)
-        af[set][mi] = *reinterpret_cast<const u32x4*>(stage + a_frag_off + mi * 32 * kRowStride + kk * 32);
+        af[set][mi] = *reinterpret_cast<const u32x4*>(stage + a_frag_off + mi * 32 * kRowBytes + xk[kk]);
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni)
-        bf[set][ni] = *reinterpret_cast<const u32x4*>(stage + b_frag_off + ni * 32 * kRowStride + kk * 32);
+        bf[set][ni] = *reinterpret_cast<const u32x4*>(stage + b_frag_off + ni * 32 * kRowBytes + xk[kk]);
     };
     auto mma = [&](int set) {
 #pragma unroll
@@ -155,7 +158,6 @@ struct GemmTile {
     constexpr int kFragReads = MI + NI;
     constexpr int kMma = MI * NI;
     constexpr int kLoads = kPassA + kPassB;
-    constexpr int kFree = kMma - kFragReads > 0 ? kMma - kFragReads : 1;   // matrix ops left after the fragment reads
     // one K-step: `kFragReads` matrix ops each followed by one LDS read, then the rest
     auto pace_reads = [&]() {
 #pragma unroll
@@ -163,80 +165,44 @@ struct GemmTile {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-    };
-    // one slab; `st` = register set holding slab s+1, `ld` = set that receives a later slab
-    auto slab_body = [&](int s, int st, int ld, char* cur, char* nxt) {
-      // K-step 0 (two sets: the loads of slab s+2 ride along here)
-      read_frags(1, cur, 1);
-      if (kSets == 2) load_slab(ld, s + 2);
-      mma(0);
-      if (kSets == 2) {
-#pragma unroll
-        for (int i = 0; i < kFragReads; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x020, (kLoads + kFragReads - 1) / kFragReads, 0);
-        }
-      } else {
-        pace_reads();
-      }
       __builtin_amdgcn_sched_group_barrier(0x008, kMma - kFragReads, 0);
-      // K-step 1
+    };
+    // one slab: `cur` holds slab s, the loads of slab s+1 into `nxt` are in flight
+    auto slab_body = [&](int s, char* cur, char* nxt) {
+      read_frags(1, cur, 1);
+      mma(0);
+      pace_reads();
       read_frags(0, cur, 2);
       mma(1);
       pace_reads();
-      __builtin_amdgcn_sched_group_barrier(0x008, kMma - kFragReads, 0);
-      // K-step 2: fragments of step 3 and the LDS stores of the next slab
       read_frags(1, cur, 3);
-      store_slab(st, nxt);
       mma(0);
       pace_reads();
-#pragma unroll
-      for (int i = 0; i < kFree; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x200, (kLoads + kFree - 1) / kFree, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x200, kLoads, 0);
       __builtin_amdgcn_sched_barrier(0);
-      // everyone has the last fragments of `cur` in registers and has written its part of `nxt`
+      // slab s+1 has landed in `nxt` for every wave; everyone holds the last fragments of `cur`
+      wait_loads();
       __syncthreads();
-      // K-step 3 covers the first fragment reads of the next slab (one set: and the next global loads)
       read_frags(0, nxt, 0);
-      if (kSets == 1) load_slab(ld, s + 2);
+      dma_slab(cur, s + 2);
       mma(1);
-      if (kSets == 1) {
 #pragma unroll
-        for (int i = 0; i < kFragReads; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x020, (kLoads + kFragReads - 1) / kFragReads, 0);
-        }
-      } else {
-        pace_reads();
+      for (int i = 0; i < kFragReads; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, (kLoads + kFragReads - 1) / kFragReads, 0);
       }
       __builtin_amdgcn_sched_group_barrier(0x008, kMma - kFragReads, 0);
       __builtin_amdgcn_sched_barrier(0);
     };
 
-    load_slab(0, 0);
-    if (kSets == 2) {
-      load_slab(1, 1);
-      store_slab(0, lds);
-      __syncthreads();
-      read_frags(0, lds, 0);
-      for (int s = 0; s < nslab; s += 2) {
-        slab_body(s, 1, 0, lds, lds + kStageBytes);
-        if (s + 1 >= nslab) break;
-        slab_body(s + 1, 0, 1, lds + kStageBytes, lds);
-      }
-    } else {
-      store_slab(0, lds);
-      load_slab(0, 1);
-      __syncthreads();
-      read_frags(0, lds, 0);
-      for (int s = 0; s < nslab; ++s)
-        slab_body(s, 0, 0, lds + (s & 1) * kStageBytes, lds + ((s & 1) ^ 1) * kStageBytes);
-    }
+    dma_slab(lds, 0);
+    wait_loads();
+    __syncthreads();
+    dma_slab(lds + kStageBytes, 1);
+    read_frags(0, lds, 0);
+    for (int s = 0; s < nslab; ++s)
+      slab_body(s, lds + (s & 1) * kStageBytes, lds + ((s & 1) ^ 1) * kStageBytes);
+    wait_loads();      // the clamped loads of the last two slabs still target LDS
     __syncthreads();   // the caller may reuse LDS; every wave is past its last fragment read
   }
 };

@@ -16,6 +16,7 @@
 namespace clgrpo {
 
 constexpr int kFwdBM = 256, kFwdBN = 256;
+constexpr int kZRow = kFwdBM * 2 + 16;   // bytes per token row of a 16-bit logits tile turned through LDS (padded)
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct FwdParams {
@@ -107,14 +108,21 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
     Tile::run(acc, weight + (int64_t)v0 * p.H, p.H, a_rows, hidden, p.H, b_rows, p.H, lds);
 
     if (STORE_Z) {
-      // Raw logits for the backward.  Vocabulary rows past V were read as zero rows of W, so the
-      // padding columns hold zeros.
+      // Raw logits for the backward; the padding columns past V are stored as zeros.
+      if (a_rows < kFwdBM) {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              if (wm * WM + mi * 32 + acc_row(r, lane) >= a_rows) acc[mi][ni][r] = 0.f;
+      }
       T* z = static_cast<T*>(p.z_out);
       typedef typename Pack4<T>::type P4;
       if (sizeof(T) == 2) {
         // 16-bit logits: turn the tile through LDS (free between two K loops) so that every token
         // row leaves as whole 16-byte pieces of one contiguous 512-byte run.
-        constexpr int kZRow = kFwdBM * 2 + 16;   // bytes per token row in LDS (padded)
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) {
           char* row = lds + (wn * WN + ni * 32 + (lane & 31)) * kZRow;
@@ -334,16 +342,19 @@ static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream) {
   p.ldz = a->ld_saved;
   p.z_row_map = a->saved_row_map;
   p.z_rows = (int)a->saved_rows;
+  // the K loop's two stages, or the logits tile when it is turned through LDS
+  constexpr int kZTile = (STORE_Z && sizeof(T) == 2) ? kFwdBN * kZRow : 0;
+  constexpr int lds_bytes = Tile::kLdsBytes > kZTile ? Tile::kLdsBytes : kZTile;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&lmhead_fwd_kernel<T, STORE_Z>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail(CLGRPO_ELAUNCH, "lmhead_fwd: LDS attribute: %s", hipGetErrorString(e));
     attr_set = true;
   }
   int grid = p.n_tb * p.n_split;
   grid = (grid + 7) / 8 * 8;
-  hipLaunchKernelGGL((lmhead_fwd_kernel<T, STORE_Z>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, p);
+  hipLaunchKernelGGL((lmhead_fwd_kernel<T, STORE_Z>), dim3(grid), dim3(Tile::kThreads), lds_bytes, stream, p);
   int rc = check_launch("lmhead_fwd_kernel");
   if (rc) return rc;
   FinalizeParams f;
