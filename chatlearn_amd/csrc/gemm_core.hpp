@@ -79,40 +79,87 @@ struct GemmTile {
   static_assert(BM % kRowsPerPass == 0 && BN % kRowsPerPass == 0, "tile rows vs threads");
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 blocks");
 
-  // acc[mi][ni] must be zeroed by the caller.  a_base/b_base point at row 0 of
-  // the tile (K offset 0).  Loads go through range-checked buffer descriptors
-  // that cover exactly the a_rows / b_rows valid rows, so rows past them read
-  // as zero and nothing outside the operands is touched.  The row part of an
-  // address always travels in the per-lane offset (the part the hardware range
-  // check is guaranteed to see); only the in-row K offset rides in the scalar
-  // offset.  K must be a multiple of kSlabK and the rows 16-byte aligned.
-  __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const T* a_base, int64_t lda,
-                                             int a_rows, const T* b_base, int64_t ldb, int b_rows,
-                                             int K, char* lds) {
+  // State a caller carries between consecutive K loops of one workgroup that share B (same
+  // token rows, next block of A rows): which LDS stage holds slab 0, and whether the first two
+  // slabs of the coming loop have already been requested.
+  struct Stream {
+    int phase = 0;
+    bool loaded = false;
+  };
+
+  // Per-thread constants of the global -> LDS loads of one operand pair.
+  struct Loader {
+    __amdgpu_buffer_rsrc_t a_rsrc, b_rsrc;
+    int a_voff, b_voff, a_pass, b_pass, dma_off;
+  };
+
+  typedef __attribute__((address_space(3))) char lds_char;
+
+  // Loads go through range-checked buffer descriptors that cover exactly the a_rows / b_rows
+  // valid rows, so rows past them read as zero and nothing outside the operands is touched.
+  // The row part of an address always travels in the per-lane offset (the part the hardware
+  // range check is guaranteed to see); only the in-row K offset rides in the scalar offset.
+  __device__ static __forceinline__ Loader make_loader(const T* a_base, int64_t lda, int a_rows,
+                                                       const T* b_base, int64_t ldb, int b_rows) {
     const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave % WAVES_M;
-    const int wn = wave / WAVES_M;
     const int ld_row = tid >> 3;
     const int ld_chunk = tid & 7;
-
     const int lda_b = (int)(lda * (int64_t)sizeof(T));
     const int ldb_b = (int)(ldb * (int64_t)sizeof(T));
-    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T*>(a_base), 0, a_rows * lda_b, 0x00020000);
-    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T*>(b_base), 0, b_rows * ldb_b, 0x00020000);
+    Loader L;
+    L.a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_base), 0, a_rows * lda_b, 0x00020000);
+    L.b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(b_base), 0, b_rows * ldb_b, 0x00020000);
     // A wave's load instruction fills 1 KB of LDS in lane order: 8 rows x 8 chunks of 16 bytes.
     // The lane that lands on (row, slot) fetches K-chunk slot ^ swz(row), so a fragment read of
     // K-chunk q goes to slot q ^ swz(row).
     const int ld_swz = (ld_row & 7) ^ ((ld_row >> 3) & 1);
-    const int a_voff = ld_row * lda_b + ((ld_chunk ^ ld_swz) * 16);
-    const int b_voff = ld_row * ldb_b + ((ld_chunk ^ ld_swz) * 16);
-    const int a_pass = kRowsPerPass * lda_b;
-    const int b_pass = kRowsPerPass * ldb_b;
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const int dma_off = wave_u * 8 * kRowBytes;   // LDS offset of this wave's 8 rows within a pass
+    L.a_voff = ld_row * lda_b + ((ld_chunk ^ ld_swz) * 16);
+    L.b_voff = ld_row * ldb_b + ((ld_chunk ^ ld_swz) * 16);
+    L.a_pass = kRowsPerPass * lda_b;
+    L.b_pass = kRowsPerPass * ldb_b;
+    L.dma_off = __builtin_amdgcn_readfirstlane(tid >> 6) * 8 * kRowBytes;   // this wave's 8 rows within a pass
+    return L;
+  }
+
+  // global -> LDS without passing registers; completion must be awaited (wait_loads) before the
+  // workgroup barrier that publishes the stage.
+  __device__ static __forceinline__ void dma_slab(const Loader& L, char* stage, int slab) {
+    const int koff = slab * kRowBytes;
+    lds_char* dst = (lds_char*)(stage) + L.dma_off;
+#pragma unroll
+    for (int p = 0; p < kPassA; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(L.a_rsrc, dst + p * kRowsPerPass * kRowBytes, 16,
+                                               L.a_voff + p * L.a_pass, koff, 0, 0);
+#pragma unroll
+    for (int p = 0; p < kPassB; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(L.b_rsrc, dst + (BM + p * kRowsPerPass) * kRowBytes, 16,
+                                               L.b_voff + p * L.b_pass, koff, 0, 0);
+  }
+
+  // A workgroup barrier does not wait for loads whose destination is LDS: wait for this wave's
+  // outstanding ones explicitly (s_waitcnt vmcnt(0), the other counters left alone).
+  __device__ static __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+  // acc[mi][ni] must be zeroed by the caller.  a_base/b_base point at row 0 of the tile (K offset
+  // 0).  K must be a multiple of kSlabK and the rows 16-byte aligned.  With a_next != nullptr the
+  // last two slab periods request the first two slabs of the next K loop (A rows from a_next, same
+  // B), and LDS stays in use on return; otherwise, with release_lds, all loads have landed and
+  // every wave is past its last fragment read on return.
+  __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const T* a_base, int64_t lda,
+                                             int a_rows, const T* b_base, int64_t ldb, int b_rows,
+                                             int K, char* lds, Stream& st, const T* a_next,
+                                             int a_next_rows, bool release_lds) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave % WAVES_M;
+    const int wn = wave / WAVES_M;
+    const Loader L = make_loader(a_base, lda, a_rows, b_base, ldb, b_rows);
+    const int nslab = K / kSlabK;
+    const bool stream_on = a_next != nullptr && nslab >= 2;
+    Loader LN = L;
+    if (stream_on)
+      LN.a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_next), 0,
+                                                    a_next_rows * (int)(lda * (int64_t)sizeof(T)), 0x00020000);
 
     const int fr_swz = (lane & 7) ^ ((lane >> 3) & 1);
     int xk[4];
@@ -121,26 +168,7 @@ struct GemmTile {
     const int a_frag_off = (wm * WM + (lane & 31)) * kRowBytes;
     const int b_frag_off = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
 
-    typedef __attribute__((address_space(3))) char lds_char;
-    const int nslab = K / kSlabK;
     u32x4 af[2][MI], bf[2][NI];
-    const int last = nslab - 1;
-    // global -> LDS without passing registers; completion is awaited before the next barrier
-    auto dma_slab = [&](char* stage, int slab) {
-      const int koff = (slab < last ? slab : last) * kRowBytes;   // clamped: always in bounds
-      lds_char* dst = (lds_char*)(stage) + dma_off;
-#pragma unroll
-      for (int p = 0; p < kPassA; ++p)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, dst + p * kRowsPerPass * kRowBytes, 16,
-                                                 a_voff + p * a_pass, koff, 0, 0);
-#pragma unroll
-      for (int p = 0; p < kPassB; ++p)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, dst + (BM + p * kRowsPerPass) * kRowBytes, 16,
-                                                 b_voff + p * b_pass, koff, 0, 0);
-    };
-    // A workgroup barrier does not wait for loads whose destination is LDS: wait for this wave's
-    // outstanding ones explicitly (s_waitcnt vmcnt(0), the other counters left alone).
-    auto wait_loads = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
     auto read_frags = [&](int set, const char* stage, int kk) {
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi)
@@ -167,8 +195,9 @@ struct GemmTile {
       }
       __builtin_amdgcn_sched_group_barrier(0x008, kMma - kFragReads, 0);
     };
-    // one slab: `cur` holds slab s, the loads of slab s+1 into `nxt` are in flight
-    auto slab_body = [&](int s, char* cur, char* nxt) {
+    // one slab: `cur` holds slab s, the loads of slab s+1 into `nxt` are in flight; `ld` and
+    // `ld_slab` name the slab requested into `cur` once everyone is done with it
+    auto slab_body = [&](char* cur, char* nxt, const Loader& ld, int ld_slab) {
       read_frags(1, cur, 1);
       mma(0);
       pace_reads();
@@ -183,7 +212,7 @@ struct GemmTile {
       wait_loads();
       __syncthreads();
       read_frags(0, nxt, 0);
-      dma_slab(cur, s + 2);
+      dma_slab(ld, cur, ld_slab);
       mma(1);
 #pragma unroll
       for (int i = 0; i < kFragReads; ++i) {
@@ -195,15 +224,40 @@ struct GemmTile {
       __builtin_amdgcn_sched_barrier(0);
     };
 
-    dma_slab(lds, 0);
-    wait_loads();
-    __syncthreads();
-    dma_slab(lds + kStageBytes, 1);
-    read_frags(0, lds, 0);
-    for (int s = 0; s < nslab; ++s)
-      slab_body(s, lds + (s & 1) * kStageBytes, lds + ((s & 1) ^ 1) * kStageBytes);
-    wait_loads();      // the clamped loads of the last two slabs still target LDS
-    __syncthreads();   // the caller may reuse LDS; every wave is past its last fragment read
+    char* const buf0 = lds + st.phase * kStageBytes;
+    char* const buf1 = lds + (st.phase ^ 1) * kStageBytes;
+    if (!st.loaded) {
+      dma_slab(L, buf0, 0);
+      wait_loads();
+      __syncthreads();
+      if (nslab > 1) dma_slab(L, buf1, 1);
+    } else {
+      wait_loads();
+      __syncthreads();
+    }
+    read_frags(0, buf0, 0);
+    int s = 0;
+    for (; s + 2 < nslab; ++s)
+      slab_body((s & 1) ? buf1 : buf0, (s & 1) ? buf0 : buf1, L, s + 2);
+    // The last two slab periods have no slab of this loop left to request: they request the first
+    // two slabs of the next loop, or the last slab again.  (Measured: leaving the loads out here
+    // instead makes the whole loop slower, not faster.)
+    for (; s < nslab; ++s)
+      slab_body((s & 1) ? buf1 : buf0, (s & 1) ? buf0 : buf1, LN, stream_on ? s + 2 - nslab : nslab - 1);
+    st.phase = (st.phase + nslab) & 1;
+    st.loaded = stream_on;
+    if (release_lds && !stream_on) {
+      wait_loads();      // the repeated loads of the last slab still target LDS
+      __syncthreads();
+    }
+  }
+
+  // Single K loop: nothing carried over, LDS free on return.
+  __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const T* a_base, int64_t lda,
+                                             int a_rows, const T* b_base, int64_t ldb, int b_rows,
+                                             int K, char* lds) {
+    Stream st;
+    run(acc, a_base, lda, a_rows, b_base, ldb, b_rows, K, lds, st, nullptr, 0, true);
   }
 };
 

@@ -92,6 +92,7 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
     zt[ni] = 0.f;
   }
 
+  typename Tile::Stream st;
   const int vt_begin = vs * p.tiles_per_split;
   const int vt_end = (vt_begin + p.tiles_per_split) < p.n_vt ? (vt_begin + p.tiles_per_split) : p.n_vt;
   for (int vt = vt_begin; vt < vt_end; ++vt) {
@@ -105,7 +106,15 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
-    Tile::run(acc, weight + (int64_t)v0 * p.H, p.H, a_rows, hidden, p.H, b_rows, p.H, lds);
+    // The K loop requests the first slabs of the next vocabulary tile during its last two slab
+    // periods, except where 16-bit logits are turned through LDS after it.
+    constexpr bool kZViaLds = STORE_Z && sizeof(T) == 2;
+    const bool has_next = vt + 1 < vt_end;
+    const int v1 = v0 + kFwdBM;
+    const int next_rows = (p.V - v1) < kFwdBM ? (p.V - v1) : kFwdBM;
+    const T* next_w = weight + (int64_t)v1 * p.H;
+    Tile::run(acc, weight + (int64_t)v0 * p.H, p.H, a_rows, hidden, p.H, b_rows, p.H, lds, st,
+              (has_next && !kZViaLds) ? next_w : nullptr, next_rows, true);
 
     if (STORE_Z) {
       // Raw logits for the backward; the padding columns past V are stored as zeros.
