@@ -32,7 +32,7 @@ PEAK_F32_TFLOPS = 157.3
 # (FETCH_SIZE scaled by 2.00, WRITE_SIZE by 1.00 after a plain 1 GiB copy calibration; the summary is
 # kept with the other profiles).  Key: (config, tokens per launch, chunk logits kept).  Other
 # workloads have not been measured and report null.
-MEASURED_FWD_TRAFFIC_BYTES = {("c2", 8192, True): 30.35e9}
+MEASURED_FWD_TRAFFIC_BYTES = {("c2", 16384, True): 49.26e9}
 
 
 def build_workload(cfg, device):
@@ -186,7 +186,7 @@ def main():
                     help="also leave rows whose loss mask is zero out of the forward (their per-token outputs become zero)")
     ap.add_argument("--no-skip-masked", action="store_true",
                     help="run the backward on every row, also those whose loss mask is zero")
-    ap.add_argument("--keep-logits-chunk", type=int, default=8192,
+    ap.add_argument("--keep-logits-chunk", type=int, default=16384,
                     help="tokens per chunk whose logits the forward keeps for the backward (0: recompute)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -277,7 +277,9 @@ def main():
 
     thv = float(T) * cfg.H * cfg.V
     peak = PEAK_BF16_TFLOPS if cfg.dtype == torch.bfloat16 else PEAK_F32_TFLOPS
-    fwd_tflops = 2.0 * thv / (fwd_ms * 1e-3) / 1e12          # all forward launches of a step together
+    # the kernel's rate counts the rows its launches projected (all T unless --skip-masked-forward)
+    fwd_flops = 2.0 * float(rows_fwd) * cfg.H * cfg.V
+    fwd_tflops = fwd_flops / (fwd_ms * 1e-3) / 1e12          # all forward launches of a step together
     step_flops = (6.0 if train else 2.0) * thv
     out = {
         "metric": "packed tokens/sec, fused logprob+GRPO loss fwd+bwd (Qwen3-8B head); % MFMA peak",
@@ -301,7 +303,7 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tflops, "peak": peak,
                      "unit": "TFLOP/s", "frac": fwd_tflops / peak,
                      "traffic": MEASURED_FWD_TRAFFIC_BYTES.get((cfg.name, max(hi - lo for lo, hi in chunks), bool(keep))),
-                     "algorithmic_flops_per_launch": 2.0 * thv / n_fwd_launch,
+                     "algorithmic_flops_per_launch": fwd_flops / n_fwd_launch,
                      "avg_launch_ms": fwd_ms / n_fwd_launch, "launches_per_step": n_fwd_launch},
         "step_mfma_frac": step_flops / dt / 1e12 / peak,
         "stage_ms": {"forward": fwd_ms, "loss": loss_ms, "backward": bwd_ms},

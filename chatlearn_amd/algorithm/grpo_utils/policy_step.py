@@ -29,7 +29,7 @@ class PolicyStep:
                  module_args: Optional[Dict[str, Any]] = None, packing: bool = False, max_token_in_seq: int = 32768,
                  train_micro_batch_size: int = 1, generate_micro_batch_size: int = 1, trainable: bool = True,
                  fsdp_size: int = 1, temperature: float = 1.0, dweight_buffer: Optional[torch.Tensor] = None,
-                 keep_logits_chunk: Optional[int] = 8192):
+                 keep_logits_chunk: Optional[int] = 16384):
         self.backbone = backbone
         self.weight = lm_head_weight
         self.module_args = dict(_DEFAULT_ARGS)

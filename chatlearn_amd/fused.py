@@ -98,7 +98,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                    pos_clip_ratio=0.2, neg_clip_ratio=0.2, diff_clip_ratio=10, final_clip_ratio=3,
                    kl_coef=0.0, entropy_coef=0.0, temperature=1.0, dweight: Optional[torch.Tensor] = None,
                    accumulate_dweight=False, need_dhidden=True, check_flags=True,
-                   keep_logits_chunk: Optional[int] = 8192, cu_seqlens_host=None, skip_masked_rows=True,
+                   keep_logits_chunk: Optional[int] = 16384, cu_seqlens_host=None, skip_masked_rows=True,
                    skip_masked_forward=False, stage_hook=None):
     """Forward + loss + backward of the head for one packed micro-batch, no autograd graph.
 
