@@ -99,7 +99,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                    kl_coef=0.0, entropy_coef=0.0, temperature=1.0, dweight: Optional[torch.Tensor] = None,
                    accumulate_dweight=False, need_dhidden=True, check_flags=True,
                    keep_logits_chunk: Optional[int] = 16384, cu_seqlens_host=None, skip_masked_rows=True,
-                   skip_masked_forward=False, stage_hook=None):
+                   skip_masked_forward=False, weight_t_cache: Optional[dict] = None, stage_hook=None):
     """Forward + loss + backward of the head for one packed micro-batch, no autograd graph.
 
     Mirrors policy_trainer.py:216-286 on packed rows: returns a dict with the
@@ -123,6 +123,10 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     them), but the returned per-token ``logprob`` / ``entropy`` / ``lse`` are zero at masked rows
     instead of the values the reference computes and then ignores; ``rows_projected_fwd`` counts
     the rows the forward ran on.
+
+    ``weight_t_cache``: a dict the caller keeps while ``weight`` does not change (the micro-batches
+    of one optimizer step).  The first backward leaves the transposed weight in it and later calls
+    reuse it instead of transposing again; the caller clears it after updating the weight.
 
     ``stage_hook(name)`` is called on the host at "forward", "loss", "backward", "end" boundaries
     of every chunk (a benchmark records stream events there).
@@ -150,8 +154,11 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     acc_dw = accumulate_dweight
     rows_projected_bwd = 0
     rows_projected_fwd = 0
-    wt = ops.weight_t_buffer(weight) if (need_dhidden and len(chunks) > 1) else None
-    wt_ready = False
+    wt, wt_ready = None, False
+    if need_dhidden and weight_t_cache is not None:
+        wt, wt_ready = weight_t_cache.get("weight_t"), weight_t_cache.get("weight_t") is not None
+    if need_dhidden and wt is None and (len(chunks) > 1 or weight_t_cache is not None):
+        wt = ops.weight_t_buffer(weight)
     kl_c = kl_coef if kl_coef > 0 else 0.0
     en_c = entropy_coef if entropy_coef > 0 else 0.0
     for lo, hi in chunks:
@@ -213,6 +220,8 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
         rows_projected_bwd += n
         hook("end")
         acc_dw = True
+        if weight_t_cache is not None and wt_ready:
+            weight_t_cache["weight_t"] = wt
         lp_all[sl], ent_all[sl], lse_all[sl], glp_all[sl], loss_all[sl] = lp, ent, lse, res.g_logprob, res.loss
         if kl_all is not None:
             kl_all[sl] = res.kl

@@ -109,3 +109,27 @@ def test_kept_logits_backward_equals_recompute(dev):
     dh2, dw2 = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_en, 0.8, saved_logits=zbuf)
     assert_close_rel(dh2, dh1, 1e-2, "dhidden kept vs recompute")
     assert_close_rel(dw2, dw1, 1e-2, "dweight kept vs recompute")
+
+
+def test_weight_transpose_cache_is_reused_across_micro_batches(dev):
+    """Two micro-batches of one optimizer step share one transposed weight: same results as
+    without the cache, the buffer object is kept, and a stale cache would be visible."""
+    from chatlearn_amd.fused import grpo_head_step
+    cfg, samples, cu, mask, T, hidden, weight, labels, old, ref, adv = _workload(CASES[1][0], dev, **CASES[1][1])
+    d = lambda x: x.to(dev)
+    kw = dict(n_tokens_total=float(mask.sum()), kl_coef=cfg.kl_coef, entropy_coef=cfg.entropy_coef,
+              temperature=cfg.temperature, cu_seqlens_host=cu.tolist())
+    args = [d(x) for x in (hidden, weight, labels, old, ref, adv, cu, mask)]
+    plain = grpo_head_step(*args, **kw)
+    cache = {}
+    first = grpo_head_step(*args, weight_t_cache=cache, **kw)
+    wt = cache["weight_t"]
+    assert torch.equal(wt[:, :weight.shape[0]], args[1].t())
+    second = grpo_head_step(*args, weight_t_cache=cache, **kw)
+    assert cache["weight_t"] is wt
+    for out in (first, second):
+        assert torch.equal(out["dhidden"], plain["dhidden"]) and torch.equal(out["dweight"], plain["dweight"])
+    # the cache is trusted: with a different weight in it the gradient follows the cached one
+    cache["weight_t"] = torch.zeros_like(wt)
+    stale = grpo_head_step(*args, weight_t_cache=cache, **kw)
+    assert (stale["dhidden"] == 0).all()
