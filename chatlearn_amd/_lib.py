@@ -96,6 +96,9 @@ SIGNATURES = {
     "clgrpo_saved_logits_ld": (i64, [i64]),
     "clgrpo_lmhead_bwd_workspace_bytes": (sz, [i64, i64, i64, i32, i64, i32]),
     "clgrpo_lmhead_bwd": (C.c_int, [C.POINTER(LmheadBwdArgs), vp]),
+    "clgrpo_lmhead_fwd_shard": (C.c_int, [C.POINTER(LmheadFwdArgs), i64, vp, vp]),
+    "clgrpo_lmhead_merge_shards": (C.c_int, [vp, i64, i64, vp, i64, f32, vp, vp, vp, vp, vp]),
+    "clgrpo_lmhead_bwd_shard": (C.c_int, [C.POINTER(LmheadBwdArgs), i64, vp]),
     "clgrpo_softmax_stats": (C.c_int, [C.POINTER(SoftmaxStatsArgs), vp]),
     "clgrpo_softmax_stats_bwd": (C.c_int, [C.POINTER(SoftmaxStatsBwdArgs), vp]),
     "clgrpo_policy_loss_workspace_bytes": (sz, [i64, i64]),

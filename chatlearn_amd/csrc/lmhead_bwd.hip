@@ -37,6 +37,7 @@ struct DzParams {
   const void* hidden;   // chunk base: [Tc, H]
   const void* weight;   // [V, H]
   const int64_t* labels;  // chunk base
+  int64_t label_offset;   // first vocabulary id of `weight` (0 unless this is a vocabulary shard)
   const float* lse;
   const float* entropy;   // or nullptr
   const float* g_lp;
@@ -79,7 +80,11 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_dz_kernel(DzParams p) {
   for (int ni = 0; ni < NI; ++ni) {
     tl[ni] = t0 + wn * WN + ni * 32 + (lane & 31);
     const bool ok = tl[ni] < p.Tc;
-    lab[ni] = ok ? (int)p.labels[tl[ni]] : -1;
+    lab[ni] = -1;
+    if (ok) {
+      const int64_t rel = p.labels[tl[ni]] - p.label_offset;   // a label outside these rows matches nothing
+      if (rel >= 0 && rel < p.V) lab[ni] = (int)rel;
+    }
     lse[ni] = ok ? p.lse[tl[ni]] : 1e30f;
     lse2[ni] = lse[ni] * kLog2e;
     glp[ni] = ok ? p.g_lp[tl[ni]] : 0.f;
@@ -146,6 +151,7 @@ struct DzFromZParams {
   void* z;            // [Tc][ldv] in: raw logits, out: dz
   void* dzT;          // [V][ldt]
   const int64_t* labels;
+  int64_t label_offset;
   const float* lse;
   const float* entropy;
   const float* g_lp;
@@ -178,7 +184,7 @@ __global__ __launch_bounds__(256) void dz_from_z_kernel(DzFromZParams p) {
         const float lse = p.lse[t];
         const float lse2 = lse * kLog2e;
         const float ent = p.g_ent ? p.entropy[t] : 0.f;
-        const int64_t lab = p.labels[t];
+        const int64_t lab = p.labels[t] - p.label_offset;
         const u32x4 raw = *reinterpret_cast<const u32x4*>(z + (int64_t)t * p.ldv + v);
         const T* in = reinterpret_cast<const T*>(&raw);
 #pragma unroll
@@ -421,7 +427,7 @@ static int launch_transpose(const T* src, int64_t ld_src, T* dst, int64_t ld_dst
 }
 
 template <typename T>
-static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream) {
+static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream, int64_t label_offset) {
   using Tile = HeadTile<T>;
   const int64_t T_ = a->T, H = a->H, V = a->V;
   const bool saved = a->saved_logits != nullptr;
@@ -460,6 +466,7 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream) {
       q.z = dz;
       q.dzT = dzt;
       q.labels = a->labels + c0;
+      q.label_offset = label_offset;
       q.lse = a->lse + c0;
       q.entropy = a->g_entropy ? a->entropy + c0 : nullptr;
       q.g_lp = a->g_logprob + c0;
@@ -479,6 +486,7 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream) {
       d.hidden = hidden + c0 * H;
       d.weight = weight;
       d.labels = a->labels + c0;
+      d.label_offset = label_offset;
       d.lse = a->lse + c0;
       d.entropy = a->g_entropy ? a->entropy + c0 : nullptr;
       d.g_lp = a->g_logprob + c0;
@@ -528,9 +536,9 @@ extern "C" size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_
   return bwd_plan(T, H, V, dtype_bytes(dtype), chunk_tokens, with_saved_logits != 0).total;
 }
 
-extern "C" int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream) {
+static int bwd_entry(const char* who, const clgrpo_lmhead_bwd_args* a, int64_t vocab_begin, void* stream) {
   CLGRPO_REQUIRE_PTR(a, "args");
-  int rc = validate_head_shape("clgrpo_lmhead_bwd", a->T, a->H, a->V, a->dtype);
+  int rc = validate_head_shape(who, a->T, a->H, a->V, a->dtype);
   if (rc) return rc;
   CLGRPO_REQUIRE_PTR(a->hidden, "hidden");
   CLGRPO_REQUIRE_PTR(a->weight, "weight");
@@ -538,13 +546,21 @@ extern "C" int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream) 
   CLGRPO_REQUIRE_PTR(a->lse, "lse");
   CLGRPO_REQUIRE_PTR(a->g_logprob, "g_logprob");
   if (a->g_entropy != nullptr) CLGRPO_REQUIRE_PTR(a->entropy, "entropy");
-  if (a->dhidden == nullptr && a->dweight == nullptr)
-    return fail(CLGRPO_ENULL, "clgrpo_lmhead_bwd: both dhidden and dweight are NULL");
-  if (!(a->inv_temperature > 0.f)) return fail(CLGRPO_EINVAL, "clgrpo_lmhead_bwd: inv_temperature must be > 0");
+  if (a->dhidden == nullptr && a->dweight == nullptr) return fail(CLGRPO_ENULL, "%s: both dhidden and dweight are NULL", who);
+  if (vocab_begin < 0) return fail(CLGRPO_EINVAL, "%s: vocab_begin=%lld", who, (long long)vocab_begin);
+  if (!(a->inv_temperature > 0.f)) return fail(CLGRPO_EINVAL, "%s: inv_temperature must be > 0", who);
   CLGRPO_REQUIRE_PTR(a->workspace, "workspace");
   if (a->saved_logits != nullptr && (a->ld_saved < round_up64(a->V, 64) || a->ld_saved % 64 != 0))
-    return fail(CLGRPO_ESHAPE, "clgrpo_lmhead_bwd: ld_saved=%lld must be a multiple of 64 and >= %lld",
-                (long long)a->ld_saved, (long long)round_up64(a->V, 64));
+    return fail(CLGRPO_ESHAPE, "%s: ld_saved=%lld must be a multiple of 64 and >= %lld", who, (long long)a->ld_saved,
+                (long long)round_up64(a->V, 64));
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return a->dtype == CLGRPO_BF16 ? run_bwd<__bf16>(a, s) : run_bwd<float>(a, s);
+  return a->dtype == CLGRPO_BF16 ? run_bwd<__bf16>(a, s, vocab_begin) : run_bwd<float>(a, s, vocab_begin);
+}
+
+extern "C" int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream) {
+  return bwd_entry("clgrpo_lmhead_bwd", a, 0, stream);
+}
+
+extern "C" int clgrpo_lmhead_bwd_shard(const clgrpo_lmhead_bwd_args* a, int64_t vocab_begin, void* stream) {
+  return bwd_entry("clgrpo_lmhead_bwd_shard", a, vocab_begin, stream);
 }

@@ -23,6 +23,7 @@ struct FwdParams {
   const void* hidden;
   const void* weight;
   const int64_t* labels;
+  int64_t label_offset;  // first vocabulary id of `weight` (0 unless this is a vocabulary shard)
   int T, H, V;
   int n_tb, n_split, tiles_per_split, n_vt;
   float c;  // inv_temperature * log2(e)
@@ -83,7 +84,11 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
     const int tok = t0 + wn * WN + ni * 32 + (lane & 31);
-    lab[ni] = (p.labels != nullptr && tok < p.T) ? (int)p.labels[tok] : -1;
+    lab[ni] = -1;
+    if (p.labels != nullptr && tok < p.T) {
+      const int64_t rel = p.labels[tok] - p.label_offset;   // a label outside these rows matches nothing
+      if (rel >= 0 && rel < p.V) lab[ni] = (int)rel;
+    }
     zrow[ni] = (STORE_Z && tok < p.T) ? (p.z_row_map ? p.z_row_map[tok] : tok) : -1;
     if (zrow[ni] >= p.z_rows) zrow[ni] = -1;
     m[ni] = -INFINITY;
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
       }
       T* z = static_cast<T*>(p.z_out);
       typedef typename Pack4<T>::type P4;
-      if (sizeof(T) == 2) {
+      if (kZViaLds) {
         // 16-bit logits: turn the tile through LDS (free between two K loops) so that every token
         // row leaves as whole 16-byte pieces of one contiguous 512-byte run.
 #pragma unroll
@@ -290,6 +295,7 @@ struct FinalizeParams {
   float* entropy;
   float* rowmax;
   float* lse;
+  float4* record;   // non-null: only the merged (max, sum, sum*z, target) record is written
 };
 
 __global__ void lmhead_fwd_finalize_kernel(FinalizeParams p) {
@@ -300,6 +306,10 @@ __global__ void lmhead_fwd_finalize_kernel(FinalizeParams p) {
     const float4 o = p.part[(int64_t)k * p.T + t];
     merge_state(m, s, u, o.x, o.y, o.z, p.c);
     zt += o.w;
+  }
+  if (p.record) {
+    p.record[t] = make_float4(m, s, u, zt);
+    return;
   }
   const float mx = m * p.inv_temperature;
   const float lse = mx + logf(s);
@@ -335,12 +345,13 @@ static void fwd_plan(int64_t T, int64_t V, int& n_tb, int& n_vt, int& n_split, i
 }
 
 template <typename T, bool STORE_Z>
-static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream) {
+static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream, int64_t label_offset, float4* record) {
   using Tile = HeadTile<T>;
   FwdParams p;
   p.hidden = a->hidden;
   p.weight = a->weight;
   p.labels = a->labels;
+  p.label_offset = label_offset;
   p.T = (int)a->T;
   p.H = (int)a->H;
   p.V = (int)a->V;
@@ -378,6 +389,7 @@ static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream) {
   f.entropy = a->entropy;
   f.rowmax = a->rowmax;
   f.lse = a->lse;
+  f.record = record;
   hipLaunchKernelGGL(lmhead_fwd_finalize_kernel, dim3((p.T + 255) / 256), dim3(256), 0, stream, f);
   return check_launch("lmhead_fwd_finalize_kernel");
 }
@@ -407,26 +419,70 @@ extern "C" size_t clgrpo_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_
   return (size_t)n_split * (size_t)T * sizeof(float4);
 }
 
-extern "C" int clgrpo_lmhead_fwd(const clgrpo_lmhead_fwd_args* a, void* stream) {
+// Shared by the whole-vocabulary entry point (record == nullptr) and the shard one.
+static int run_fwd(const char* who, const clgrpo_lmhead_fwd_args* a, int64_t vocab_begin, float4* record,
+                   void* stream) {
   CLGRPO_REQUIRE_PTR(a, "args");
-  int rc = validate_head_shape("clgrpo_lmhead_fwd", a->T, a->H, a->V, a->dtype);
+  int rc = validate_head_shape(who, a->T, a->H, a->V, a->dtype);
   if (rc) return rc;
   CLGRPO_REQUIRE_PTR(a->hidden, "hidden");
   CLGRPO_REQUIRE_PTR(a->weight, "weight");
-  CLGRPO_REQUIRE_PTR(a->lse, "lse");
-  if (a->labels != nullptr) CLGRPO_REQUIRE_PTR(a->logprob, "logprob");
-  if (!(a->inv_temperature > 0.f)) return fail(CLGRPO_EINVAL, "clgrpo_lmhead_fwd: inv_temperature must be > 0");
+  if (record == nullptr) {
+    CLGRPO_REQUIRE_PTR(a->lse, "lse");
+    if (a->labels != nullptr) CLGRPO_REQUIRE_PTR(a->logprob, "logprob");
+  }
+  if (vocab_begin < 0) return fail(CLGRPO_EINVAL, "%s: vocab_begin=%lld", who, (long long)vocab_begin);
+  if (!(a->inv_temperature > 0.f)) return fail(CLGRPO_EINVAL, "%s: inv_temperature must be > 0", who);
   CLGRPO_REQUIRE_PTR(a->workspace, "workspace");
   const size_t need = clgrpo_lmhead_fwd_workspace_bytes(a->T, a->H, a->V, a->dtype);
   if (a->workspace_bytes < need)
-    return fail(CLGRPO_EWORKSPACE, "clgrpo_lmhead_fwd: workspace %zu < %zu bytes", a->workspace_bytes, need);
+    return fail(CLGRPO_EWORKSPACE, "%s: workspace %zu < %zu bytes", who, a->workspace_bytes, need);
   if (a->saved_logits != nullptr && (a->ld_saved < clgrpo_saved_logits_ld(a->V) || a->ld_saved % 64 != 0))
-    return fail(CLGRPO_ESHAPE, "clgrpo_lmhead_fwd: ld_saved=%lld must be a multiple of 64 and >= %lld",
+    return fail(CLGRPO_ESHAPE, "%s: ld_saved=%lld must be a multiple of 64 and >= %lld", who,
                 (long long)a->ld_saved, (long long)clgrpo_saved_logits_ld(a->V));
   if (a->saved_logits != nullptr && (a->saved_rows <= 0 || a->saved_rows >= (1LL << 31)))
-    return fail(CLGRPO_EINVAL, "clgrpo_lmhead_fwd: saved_rows=%lld", (long long)a->saved_rows);
+    return fail(CLGRPO_EINVAL, "%s: saved_rows=%lld", who, (long long)a->saved_rows);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (a->saved_logits != nullptr)
-    return a->dtype == CLGRPO_BF16 ? launch_fwd<__bf16, true>(a, s) : launch_fwd<float, true>(a, s);
-  return a->dtype == CLGRPO_BF16 ? launch_fwd<__bf16, false>(a, s) : launch_fwd<float, false>(a, s);
+    return a->dtype == CLGRPO_BF16 ? launch_fwd<__bf16, true>(a, s, vocab_begin, record)
+                                   : launch_fwd<float, true>(a, s, vocab_begin, record);
+  return a->dtype == CLGRPO_BF16 ? launch_fwd<__bf16, false>(a, s, vocab_begin, record)
+                                 : launch_fwd<float, false>(a, s, vocab_begin, record);
+}
+
+extern "C" int clgrpo_lmhead_fwd(const clgrpo_lmhead_fwd_args* a, void* stream) {
+  return run_fwd("clgrpo_lmhead_fwd", a, 0, nullptr, stream);
+}
+
+extern "C" int clgrpo_lmhead_fwd_shard(const clgrpo_lmhead_fwd_args* a, int64_t vocab_begin, void* record,
+                                       void* stream) {
+  CLGRPO_REQUIRE_PTR(record, "record");
+  return run_fwd("clgrpo_lmhead_fwd_shard", a, vocab_begin, static_cast<float4*>(record), stream);
+}
+
+extern "C" int clgrpo_lmhead_merge_shards(const void* records, int64_t n_shards, int64_t T, const int64_t* labels,
+                                          int64_t V_total, float inv_temperature, float* logprob, float* entropy,
+                                          float* rowmax, float* lse, void* stream) {
+  CLGRPO_REQUIRE_PTR(records, "records");
+  CLGRPO_REQUIRE_PTR(lse, "lse");
+  if (labels != nullptr) CLGRPO_REQUIRE_PTR(logprob, "logprob");
+  if (n_shards <= 0 || n_shards > 4096 || T <= 0 || T >= (1LL << 30) || V_total <= 0)
+    return fail(CLGRPO_EINVAL, "clgrpo_lmhead_merge_shards: n_shards=%lld T=%lld V_total=%lld", (long long)n_shards,
+                (long long)T, (long long)V_total);
+  if (!(inv_temperature > 0.f)) return fail(CLGRPO_EINVAL, "clgrpo_lmhead_merge_shards: inv_temperature must be > 0");
+  FinalizeParams f;
+  f.part = static_cast<const float4*>(records);
+  f.labels = labels;
+  f.T = (int)T;
+  f.V = (int)(V_total < (1LL << 31) - 1 ? V_total : (1LL << 31) - 1);
+  f.n_split = (int)n_shards;
+  f.c = inv_temperature * kLog2e;
+  f.inv_temperature = inv_temperature;
+  f.logprob = labels ? logprob : nullptr;
+  f.entropy = entropy;
+  f.rowmax = rowmax;
+  f.lse = lse;
+  f.record = nullptr;
+  hipLaunchKernelGGL(lmhead_fwd_finalize_kernel, dim3((f.T + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), f);
+  return check_launch("lmhead_fwd_finalize_kernel");
 }

@@ -58,7 +58,8 @@ def weight_t_buffer(weight: torch.Tensor) -> torch.Tensor:
 
 def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[torch.Tensor],
                    temperature: float = 1.0, need_entropy: bool = True,
-                   saved_logits: Optional[torch.Tensor] = None, saved_row_map: Optional[torch.Tensor] = None
+                   saved_logits: Optional[torch.Tensor] = None, saved_row_map: Optional[torch.Tensor] = None,
+                   _shard_begin: Optional[int] = None
                    ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], torch.Tensor, torch.Tensor]:
     """(logprob, entropy, rowmax, lse), each fp32 [T].  Logits are not materialised unless the caller
     hands in ``saved_logits`` (from ``saved_logits_buffer``) for these T rows, which a following
@@ -76,12 +77,18 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
             raise ValueError(f"labels must have {T} elements, got {labels.numel()}")
     dt = _dtype_enum(hidden)
     f = dict(dtype=torch.float32, device=hidden.device)
-    lse = torch.empty(T, **f)
-    rowmax = torch.empty(T, **f)
-    logprob = torch.empty(T, **f) if labels is not None else None
-    entropy = torch.empty(T, **f) if need_entropy else None
-    if T == 0:
-        return logprob, entropy, rowmax, lse
+    if _shard_begin is not None:
+        record = torch.empty(T, 4, **f)
+        lse = rowmax = logprob = entropy = None
+        if T == 0:
+            return record
+    else:
+        lse = torch.empty(T, **f)
+        rowmax = torch.empty(T, **f)
+        logprob = torch.empty(T, **f) if labels is not None else None
+        entropy = torch.empty(T, **f) if need_entropy else None
+        if T == 0:
+            return logprob, entropy, rowmax, lse
     ws_bytes = _lib.lib().clgrpo_lmhead_fwd_workspace_bytes(T, H, V, dt)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=hidden.device)
     ld_saved = 0
@@ -100,7 +107,49 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
                            _ptr(logprob), _ptr(entropy), _ptr(rowmax), _ptr(lse), _ptr(ws), ws.numel(),
                            _ptr(saved_logits), ld_saved, _ptr(saved_row_map) if saved_logits is not None else None,
                            saved_logits.shape[0] if saved_logits is not None else 0)
+    if _shard_begin is not None:
+        _lib.check(_lib.lib().clgrpo_lmhead_fwd_shard(_lib.C.byref(a), int(_shard_begin), _ptr(record),
+                                                      _lib.vp(_stream(hidden) or 0)))
+        return record
     _lib.call("clgrpo_lmhead_fwd", a, _stream(hidden))
+    return logprob, entropy, rowmax, lse
+
+
+def lmhead_forward_shard(hidden: torch.Tensor, weight_shard: torch.Tensor, labels: Optional[torch.Tensor],
+                         vocab_begin: int, temperature: float = 1.0,
+                         saved_logits: Optional[torch.Tensor] = None,
+                         saved_row_map: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One vocabulary shard of the head: ``weight_shard`` holds rows ``[vocab_begin, vocab_begin + Vs)``
+    of the full matrix, ``labels`` are global ids.  Returns the per-token record fp32 [T, 4] =
+    (max raw logit, sum 2^((z-max)c), sum 2^((z-max)c)*z, target logit or 0) that
+    ``lmhead_merge_shards`` combines across shards."""
+    return lmhead_forward(hidden, weight_shard, labels, temperature, True, saved_logits, saved_row_map,
+                          _shard_begin=int(vocab_begin))
+
+
+def lmhead_merge_shards(records: torch.Tensor, labels: Optional[torch.Tensor], vocab_size: int,
+                        temperature: float = 1.0, need_entropy: bool = True):
+    """Merge the records of all vocabulary shards ([n_shards, T, 4], e.g. after an all-gather over
+    the tensor-parallel group) into (logprob, entropy, rowmax, lse), each fp32 [T]."""
+    records = _dev(records, "records", torch.float32)
+    if records.dim() != 3 or records.shape[2] != 4:
+        raise ValueError(f"records must be [n_shards, T, 4], got {tuple(records.shape)}")
+    n, T = records.shape[0], records.shape[1]
+    if labels is not None:
+        labels = _dev(labels, "labels", torch.int64)
+        if labels.numel() != T:
+            raise ValueError(f"labels must have {T} elements, got {labels.numel()}")
+    f = dict(dtype=torch.float32, device=records.device)
+    lse, rowmax = torch.empty(T, **f), torch.empty(T, **f)
+    logprob = torch.empty(T, **f) if labels is not None else None
+    entropy = torch.empty(T, **f) if need_entropy else None
+    if T == 0:
+        return logprob, entropy, rowmax, lse
+    if n == 0:
+        raise ValueError("at least one shard is needed")
+    _lib.check(_lib.lib().clgrpo_lmhead_merge_shards(_ptr(records), n, T, _ptr(labels), int(vocab_size),
+                                                     1.0 / float(temperature), _ptr(logprob), _ptr(entropy),
+                                                     _ptr(rowmax), _ptr(lse), _lib.vp(_stream(records) or 0)))
     return logprob, entropy, rowmax, lse
 
 
@@ -109,12 +158,15 @@ def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=N
                     accumulate_dweight=False, chunk_tokens: Optional[int] = None,
                     max_workspace_bytes: int = DEFAULT_BWD_WORKSPACE_BYTES,
                     saved_logits: Optional[torch.Tensor] = None, weight_t: Optional[torch.Tensor] = None,
-                    weight_t_ready: bool = False):
+                    weight_t_ready: bool = False, vocab_begin: int = 0):
     """(dhidden [T,H] in hidden's dtype, dweight [V,H] fp32).  ``dweight`` may be a caller
     buffer (e.g. the fp32 main-grad) that is overwritten or, with ``accumulate_dweight``, added to.
     ``saved_logits``: the buffer the forward of these rows filled; it is overwritten with d(logits).
     ``weight_t`` (from ``weight_t_buffer``) keeps W^T between calls that share the weight; pass
-    ``weight_t_ready=True`` once a call has filled it."""
+    ``weight_t_ready=True`` once a call has filled it.  ``vocab_begin`` > 0 (or a weight that is a
+    vocabulary shard starting at 0): ``weight`` holds rows ``[vocab_begin, vocab_begin + V)`` of the full
+    matrix, ``labels`` are global ids, ``lse`` / ``entropy`` the merged ones of all shards; ``dweight`` is
+    then this shard's rows and ``dhidden`` its partial sum."""
     hidden = _dev(hidden, "hidden")
     weight = _dev(weight, "weight", hidden.dtype)
     labels = _dev(labels, "labels", torch.int64)
@@ -168,7 +220,10 @@ def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=N
                            _ptr(g_entropy), T, H, V, dt, 1.0 / float(temperature), _ptr(dhidden), _ptr(dweight),
                            1 if accumulate_dweight else 0, _ptr(ws), ws.numel(), _ptr(saved_logits), ld_saved,
                            _ptr(weight_t), 1 if (weight_t is not None and weight_t_ready) else 0)
-    _lib.call("clgrpo_lmhead_bwd", a, _stream(hidden))
+    if vocab_begin:
+        _lib.check(L.clgrpo_lmhead_bwd_shard(_lib.C.byref(a), int(vocab_begin), _lib.vp(_stream(hidden) or 0)))
+    else:
+        _lib.call("clgrpo_lmhead_bwd", a, _stream(hidden))
     return dhidden, dweight
 
 

@@ -114,6 +114,31 @@ size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_
 int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream);
 
 /* ------------------------------------------------------------------ *
+ * One vocabulary shard of the head (tensor-parallel lm_head: each rank keeps rows
+ * [vocab_begin, vocab_begin + V) of the weight).  Replaces, per rank, the local part of
+ * Megatron's vocab-parallel cross entropy and of _VocabParallelEntropy
+ * (megatron_utils/train_helper.py:605-627): instead of three all-reduces over [T] (max,
+ * sum of exponentials, sum of p*z) plus the target-logit reduce, a rank produces one 16-byte
+ * record per token; the records of all ranks (exchanged by the caller) are merged exactly.
+ *
+ *   record[t] = (max_v z, sum_v 2^((z-max)*c), sum_v 2^((z-max)*c) * z, z[label] if the label
+ *                falls in this shard else 0),   z = raw shard logits, c = log2(e) * inv_temperature
+ *
+ * clgrpo_lmhead_fwd_shard: `a` as for clgrpo_lmhead_fwd with V = rows of this shard and GLOBAL label
+ * ids; a->logprob / entropy / rowmax / lse are ignored (may be NULL); saved_logits keeps the shard's
+ * logits as usual.  clgrpo_lmhead_merge_shards: records laid out [n_shards][T]; V_total bounds the
+ * labels (outside => NaN logprob).  clgrpo_lmhead_bwd_shard: `a` as for clgrpo_lmhead_bwd with the
+ * shard's weight and V, GLOBAL labels, and the merged lse / entropy; dweight is the shard's rows,
+ * dhidden this shard's partial sum (the caller adds the shards').
+ * ------------------------------------------------------------------ */
+int clgrpo_lmhead_fwd_shard(const clgrpo_lmhead_fwd_args* a, int64_t vocab_begin, void* record /* float4 [T] */,
+                            void* stream);
+int clgrpo_lmhead_merge_shards(const void* records, int64_t n_shards, int64_t T, const int64_t* labels,
+                               int64_t V_total, float inv_temperature, float* logprob, float* entropy,
+                               float* rowmax, float* lse, void* stream);
+int clgrpo_lmhead_bwd_shard(const clgrpo_lmhead_bwd_args* a, int64_t vocab_begin, void* stream);
+
+/* ------------------------------------------------------------------ *
  * Softmax statistics from materialised logits (legacy call sites that already
  * hold [R, V] logits) and the matching backward.
  * Replaces: logprobs_from_logits, entropy_from_logits, entropy_from_logits_with_chunking,

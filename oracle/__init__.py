@@ -23,4 +23,8 @@ of them, so none is pinned by a reference fixture):
   round-trip ``pad(unpad(x)) == x * mask``.
 * group advantages: ``numpy.mean`` / ``numpy.std`` and the Bernoulli closed
   form ``(1-k/G)/(sqrt(k/G(1-k/G))+1e-5)``.
+* vocabulary-parallel logprob / entropy (the reference's three all-reduces
+  over tensor-parallel ranks): equality with the unsharded log_softmax gather
+  and entropy for every way of cutting the vocabulary, and the uniform-logits
+  closed form.
 """

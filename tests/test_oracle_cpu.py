@@ -290,3 +290,26 @@ def test_advantage_carry_over_and_numpy_semantics():
     pool = [0.25, 1.0, 0.5, 0.0]
     assert second[0]["advantages"] == (0.5 - np.mean(pool)) / (np.std(pool) + 1e-5)   # ddof = 0, eps 1e-5
     assert "7_1" not in ac.rule_reward_buffer
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 6])
+def test_vocab_parallel_oracle_equals_unsharded_for_any_split(n):
+    """The rank-by-rank reductions (max, sum of exponentials, masked target gather, sum of p*z)
+    must give the plain log_softmax gather and entropy however the vocabulary is cut; a wrong
+    sign, a gather outside the owner's range or a missing max shift breaks one of them."""
+    from oracle import vocab_parallel as ovp
+    g = torch.Generator().manual_seed(n)
+    z = torch.randn(9, 24, generator=g, dtype=torch.float64) * 4
+    labels = torch.randint(0, 24, (9,), generator=g)
+    labels[0], labels[1] = 0, 23
+    ranges = ovp.shard_ranges(24, n)
+    shards = [z[:, lo:hi] for lo, hi in ranges]
+    assert torch.allclose(ovp.vocab_parallel_logprob(shards, labels, ranges).double(),
+                          torch.log_softmax(z, -1).gather(1, labels[:, None]).squeeze(1), atol=1e-5)
+    p = torch.softmax(z, -1)
+    assert torch.allclose(ovp.vocab_parallel_entropy(shards).double(), -(p * p.log()).sum(-1), atol=1e-5)
+    # uniform logits: entropy log V, logprob -log V whichever rank owns the label
+    u = [torch.zeros(3, 24 // n) for _ in range(n)]
+    assert torch.allclose(ovp.vocab_parallel_entropy(u), torch.full((3,), math.log(24.0)))
+    assert torch.allclose(ovp.vocab_parallel_logprob(u, torch.tensor([0, 11, 23]), ranges),
+                          torch.full((3,), -math.log(24.0)))
