@@ -83,6 +83,13 @@ class UnpadIndicesArgs(C.Structure):
                 ("seqlens", vp), ("total", vp), ("row_offsets", vp)]
 
 
+class ThdPackArgs(C.Structure):
+    _fields_ = [("B", i64), ("S", i64), ("tokens", vp), ("prompt_len", vp), ("response_len", vp),
+                ("align", i32), ("cp_size", i32), ("cp_rank", i32), ("pad_token", i64), ("total_padded", i64),
+                ("cu_seqlens_padded", vp), ("seqlens", vp), ("seqlens_padded", vp), ("stats", vp), ("status", vp),
+                ("indices", vp), ("seq_indices", vp), ("out_tokens", vp), ("out_labels", vp), ("out_loss_mask", vp)]
+
+
 class RowsArgs(C.Structure):
     _fields_ = [("src", vp), ("dst", vp), ("indices", vp), ("n_idx", i64), ("row_bytes", i64), ("n_rows", i64)]
 
@@ -107,6 +114,7 @@ SIGNATURES = {
     "clgrpo_build_masks": (C.c_int, [C.POINTER(BuildMasksArgs), vp]),
     "clgrpo_shift_labels": (C.c_int, [C.POINTER(ShiftLabelsArgs), vp]),
     "clgrpo_unpad_indices": (C.c_int, [C.POINTER(UnpadIndicesArgs), vp]),
+    "clgrpo_thd_pack": (C.c_int, [C.POINTER(ThdPackArgs), vp]),
     "clgrpo_gather_rows": (C.c_int, [C.POINTER(RowsArgs), vp]),
     "clgrpo_scatter_rows": (C.c_int, [C.POINTER(RowsArgs), vp]),
     "clgrpo_bin_packing": (C.c_int, [vp, i64, i64, vp, vp, vp]),

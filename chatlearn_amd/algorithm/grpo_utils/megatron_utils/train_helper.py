@@ -3,11 +3,15 @@ for one tensor-parallel and one context-parallel rank: the per-token logprob tha
 Megatron's vocab-parallel cross entropy yields, the vocab-parallel entropy, the
 re-padding of packed outputs, ``_compute_all_losses`` and ``loss_func``.
 
-The reference's ``get_batch`` / ``forward_step`` (Megatron and Transformer-Engine
-plumbing) are not mirrored; the functions here start where the model has produced
-``all_token_logits`` in Megatron's ``[s, b, V]`` (or ``[total_nnz, 1, V]``) layout.
+Of the reference's ``get_batch`` only the packed (THD) branch is mirrored, as
+``get_batch_packed``: one device pass replaces its per-sample Python loops.  The dense
+branch ([1, 1, S, S] attention masks, position-id resets) and ``forward_step`` are
+Megatron plumbing and stay with the caller; the loss functions here start where the
+model has produced ``all_token_logits`` in Megatron's ``[s, b, V]`` (or
+``[total_nnz, 1, V]``) layout.
 """
-from typing import Any, Dict
+from dataclasses import dataclass
+from typing import Any, Dict, Optional
 
 import torch
 
@@ -15,6 +19,67 @@ from .... import ops
 from ....bert_padding import pad_input
 from ..loss_gallery import calculate_gspo_loss, calculate_grpo_loss
 from ..trainer_utils import _StatsFromLogits
+
+
+@dataclass
+class PackedSeqParams:
+    """Field-for-field stand-in for ``megatron.core.packed_seq_params.PackedSeqParams`` as the
+    reference fills it (train_helper.py:304-310)."""
+    qkv_format: str = 'thd'
+    cu_seqlens_q: Optional[torch.Tensor] = None
+    cu_seqlens_kv: Optional[torch.Tensor] = None
+    max_seqlen_q: Optional[int] = None
+    max_seqlen_kv: Optional[int] = None
+
+
+def get_batch_packed(data_b: Dict[str, Any], is_training: bool, *, eod: int, tp_size: int = 1, cp_size: int = 1,
+                     cp_rank: int = 0, device=None) -> Dict[str, Any]:
+    """The packed branch of the reference's ``get_batch`` (train_helper.py:258-328, 400-420) for one
+    raw batch ``data_b`` (``all_tokens`` [mbs, seq_length], ``prompt_token_length``,
+    ``response_token_length``; for training also ``ref_logprobs``, ``old_logprobs``, ``advantages``
+    and optionally ``loss_mask``).  Same keys and shapes as the reference returns; the sequence
+    padding to ``tp*cp*2``, the unpadding, the label roll, the rolled packed loss mask and this
+    context-parallel rank's share come from one device pass instead of O(mbs) Python loops."""
+    tokens = data_b["all_tokens"].long()
+    device = device or (tokens.device if tokens.is_cuda else torch.device("cuda", torch.cuda.current_device()))
+    tokens = tokens.to(device)
+    mbs, seqlen = tokens.shape
+    packed = ops.thd_pack(tokens, data_b["prompt_token_length"], data_b["response_token_length"],
+                          align=tp_size * cp_size * 2, pad_token=eod, cp_size=cp_size, cp_rank=cp_rank)
+    max_padded = packed["max_seqlen_padded"]
+    params = PackedSeqParams(qkv_format='thd', cu_seqlens_q=packed["cu_seqlens_padded"],
+                             cu_seqlens_kv=packed["cu_seqlens_padded"], max_seqlen_q=max_padded,
+                             max_seqlen_kv=max_padded)
+    input_data = {
+        "all_tokens": packed["tokens"].unsqueeze(0),
+        "all_token_attention_mask": None,
+        "all_token_loss_mask": None,
+        "all_token_position_ids": None,
+        "labels": packed["labels"].unsqueeze(0),
+        'packed_seq_params': params,
+        "ori_seq_len": max_padded,
+        "ori_batch_size": mbs,
+        "seq_indices": packed["seq_indices"].unsqueeze(0),
+        "indices": packed["indices"],
+        "num_tokens_on_this_cp_rank": packed["num_loss_tokens"],
+        'pad_size': max_padded - seqlen,
+    }
+    if is_training:
+        if "loss_mask" in data_b:
+            loss_mask = data_b['loss_mask'].to(device).to(torch.int32).contiguous()
+        else:
+            as_i32 = lambda x: torch.as_tensor(x, dtype=torch.int32).to(device)
+            _, loss_mask, _ = ops.build_masks(as_i32(data_b["prompt_token_length"]),
+                                              as_i32(data_b["response_token_length"]), seqlen,
+                                              want_position_ids=False)
+        _, loss_mask = ops.shift_labels(None, loss_mask, zero_last=False)      # roll by -1 along the row
+        input_data.update({
+            "all_token_loss_mask": loss_mask,
+            "advantages": data_b["advantages"],
+            "ref_logprobs": data_b["ref_logprobs"].float().to(device),
+            "old_logprobs": data_b["old_logprobs"].float().to(device),
+        })
+    return input_data
 
 
 def language_model_logprob(labels: torch.Tensor, logits: torch.Tensor) -> torch.Tensor:

@@ -151,6 +151,133 @@ static int rows_dispatch(const clgrpo_rows_args* a, hipStream_t s, int scatter) 
   return check_launch("gather_rows_kernel");
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Packed (THD) micro-batch from per-sample lengths.
+
+// One workgroup: padded lengths, their exclusive scan, totals and the consistency word.
+__global__ __launch_bounds__(256) void thd_offsets_kernel(int64_t B, int64_t S, const int32_t* __restrict__ plen,
+                                                          const int32_t* __restrict__ rlen, int align, int cp_size,
+                                                          int64_t total_expected, int32_t* __restrict__ cu,
+                                                          int32_t* __restrict__ seqlens, int32_t* __restrict__ padded,
+                                                          int32_t* __restrict__ stats, int32_t* __restrict__ status) {
+  __shared__ int64_t part[256];
+  __shared__ int32_t pmax[256];
+  __shared__ int32_t bad[256];
+  const int tid = threadIdx.x;
+  const int64_t per = (B + 255) / 256;
+  const int64_t lo = tid * per, hi = (lo + per) < B ? (lo + per) : B;
+  int64_t sum = 0;
+  int32_t mx = 0, flag = 0;
+  for (int64_t b = lo; b < hi; ++b) {
+    const int64_t len = (int64_t)plen[b] + rlen[b];
+    const int64_t pad = (len + align - 1) / align * align;
+    seqlens[b] = (int32_t)len;
+    padded[b] = (int32_t)pad;
+    if (len > S || len < 0) flag |= 2;
+    if (pad % (2 * cp_size) != 0) flag |= 4;
+    sum += pad;
+    mx = pad > mx ? (int32_t)pad : mx;
+  }
+  part[tid] = sum;
+  pmax[tid] = mx;
+  bad[tid] = flag;
+  __syncthreads();
+  if (tid == 0) {
+    int64_t run = 0;
+    int32_t m = 0, f = 0;
+    for (int i = 0; i < 256; ++i) {
+      const int64_t v = part[i];
+      part[i] = run;
+      run += v;
+      m = pmax[i] > m ? pmax[i] : m;
+      f |= bad[i];
+    }
+    if (run != total_expected) f |= 1;
+    cu[B] = (int32_t)run;
+    stats[0] = (int32_t)run;
+    stats[1] = m;
+    stats[2] = 0;
+    status[0] = f;
+  }
+  __syncthreads();
+  int64_t run = part[tid];
+  for (int64_t b = lo; b < hi; ++b) {
+    cu[b] = (int32_t)run;
+    run += padded[b];
+  }
+}
+
+// Largest i with cu[i] <= pos (cu ascending, cu[0] = 0, pos < cu[B]; empty segments are skipped).
+__device__ __forceinline__ int thd_find_seq(const int32_t* __restrict__ cu, int B, int64_t pos) {
+  int lo = 0, hi = B;   // invariant: cu[lo] <= pos < cu[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu[mid] <= pos) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+struct ThdFill {
+  int64_t B, S, total, per_rank;
+  const int64_t* tokens;
+  const int32_t* plen;
+  const int32_t* rlen;
+  const int32_t* cu;
+  const int32_t* seqlens;
+  const int32_t* status;
+  int32_t* stats;
+  int cp_size, cp_rank;
+  int64_t pad_token;
+  int64_t* indices;
+  int64_t* seq_indices;
+  int64_t* out_tokens;
+  int64_t* out_labels;
+  int32_t* out_loss_mask;
+};
+
+__device__ __forceinline__ void thd_at(const ThdFill& p, int64_t pos, int64_t& token, int& in_loss, int& seq, int64_t& j) {
+  seq = thd_find_seq(p.cu, (int)p.B, pos);
+  j = pos - p.cu[seq];
+  token = j < p.seqlens[seq] ? p.tokens[(int64_t)seq * p.S + j] : p.pad_token;
+  const int64_t pl = p.plen[seq];
+  in_loss = (j >= pl && j < pl + p.rlen[seq]) ? 1 : 0;
+}
+
+__global__ __launch_bounds__(256) void thd_fill_kernel(ThdFill p) {
+  if (p.status[0] != 0) return;   // inconsistent sizes: leave the outputs alone, the host raises
+  const int max_padded = p.stats[1];
+  int ones = 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < p.total; i += (int64_t)gridDim.x * blockDim.x) {
+    int64_t token, j;
+    int in_loss, seq;
+    thd_at(p, i, token, in_loss, seq, j);
+    p.indices[i] = (int64_t)seq * max_padded + j;
+    if (i < p.per_rank) {
+      // i-th entry of this rank: position `src` of the packed row
+      const int sq = thd_find_seq(p.cu, (int)p.B, i * p.cp_size);   // the rank's share keeps the order of the sequences
+      const int64_t start_r = p.cu[sq] / p.cp_size;
+      const int64_t len_r = (p.cu[sq + 1] - p.cu[sq]) / p.cp_size;
+      const int64_t k = i - start_r;
+      const int64_t half = len_r / 2;
+      const int64_t chunk = k < half ? p.cp_rank : 2 * (p.cp_size - 1) - p.cp_rank;
+      const int64_t src = (int64_t)p.cu[sq] + k + half * chunk;
+      p.seq_indices[i] = src;
+      int64_t tk, nj;
+      int il, ns;
+      thd_at(p, src, tk, il, ns, nj);
+      p.out_tokens[i] = tk;
+      thd_at(p, src + 1 == p.total ? 0 : src + 1, tk, il, ns, nj);
+      p.out_labels[i] = tk;
+      if (p.out_loss_mask) p.out_loss_mask[i] = il;
+      ones += il;
+    }
+  }
+  // number of loss positions on this rank: wave reduction, one atomic per wave
+  for (int off = 32; off > 0; off >>= 1) ones += __shfl_down(ones, off, 64);
+  if ((threadIdx.x & 63) == 0 && ones) atomicAdd(&p.stats[2], ones);
+}
+
 }  // namespace clgrpo
 
 using namespace clgrpo;
@@ -231,4 +358,54 @@ extern "C" int clgrpo_scatter_rows(const clgrpo_rows_args* a, void* stream) {
     if (rc) return rc;
   }
   return rows_dispatch(a, s, 1);
+}
+
+extern "C" int clgrpo_thd_pack(const clgrpo_thd_pack_args* a, void* stream) {
+  CLGRPO_REQUIRE_PTR(a, "args");
+  if (a->B <= 0 || a->S <= 0) return fail(CLGRPO_EINVAL, "clgrpo_thd_pack: B=%lld S=%lld", (long long)a->B, (long long)a->S);
+  if (a->align <= 0 || a->cp_size <= 0 || a->cp_rank < 0 || a->cp_rank >= a->cp_size)
+    return fail(CLGRPO_EINVAL, "clgrpo_thd_pack: align=%d cp_size=%d cp_rank=%d", a->align, a->cp_size, a->cp_rank);
+  if (a->total_padded <= 0 || a->total_padded >= (1LL << 31) || a->total_padded % a->cp_size != 0)
+    return fail(CLGRPO_EINVAL, "clgrpo_thd_pack: total_padded=%lld must be positive, fit int32 and divide by cp_size",
+                (long long)a->total_padded);
+  if (a->B >= (1LL << 24)) return fail(CLGRPO_ESHAPE, "clgrpo_thd_pack: B too large");
+  CLGRPO_REQUIRE_PTR(a->tokens, "tokens");
+  CLGRPO_REQUIRE_PTR(a->prompt_len, "prompt_len");
+  CLGRPO_REQUIRE_PTR(a->response_len, "response_len");
+  CLGRPO_REQUIRE_PTR(a->cu_seqlens_padded, "cu_seqlens_padded");
+  CLGRPO_REQUIRE_PTR(a->seqlens, "seqlens");
+  CLGRPO_REQUIRE_PTR(a->seqlens_padded, "seqlens_padded");
+  CLGRPO_REQUIRE_PTR(a->stats, "stats");
+  CLGRPO_REQUIRE_PTR(a->status, "status");
+  CLGRPO_REQUIRE_PTR(a->indices, "indices");
+  CLGRPO_REQUIRE_PTR(a->seq_indices, "seq_indices");
+  CLGRPO_REQUIRE_PTR(a->out_tokens, "out_tokens");
+  CLGRPO_REQUIRE_PTR(a->out_labels, "out_labels");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(thd_offsets_kernel, dim3(1), dim3(256), 0, s, a->B, a->S, a->prompt_len, a->response_len, a->align,
+                     a->cp_size, a->total_padded, a->cu_seqlens_padded, a->seqlens, a->seqlens_padded, a->stats, a->status);
+  int rc = check_launch("thd_offsets_kernel");
+  if (rc) return rc;
+  ThdFill f;
+  f.B = a->B;
+  f.S = a->S;
+  f.total = a->total_padded;
+  f.per_rank = a->total_padded / a->cp_size;
+  f.tokens = a->tokens;
+  f.plen = a->prompt_len;
+  f.rlen = a->response_len;
+  f.cu = a->cu_seqlens_padded;
+  f.seqlens = a->seqlens;
+  f.status = a->status;
+  f.stats = a->stats;
+  f.cp_size = a->cp_size;
+  f.cp_rank = a->cp_rank;
+  f.pad_token = a->pad_token;
+  f.indices = a->indices;
+  f.seq_indices = a->seq_indices;
+  f.out_tokens = a->out_tokens;
+  f.out_labels = a->out_labels;
+  f.out_loss_mask = a->out_loss_mask;
+  hipLaunchKernelGGL(thd_fill_kernel, dim3(grid_for(a->total_padded, 256)), dim3(256), 0, s, f);
+  return check_launch("thd_fill_kernel");
 }

@@ -5,7 +5,7 @@ Every function here requires device tensors and the built library; nothing
 falls back to torch arithmetic.
 """
 import ctypes as C
-from typing import List, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
@@ -421,6 +421,55 @@ def unpad_indices(attn_mask: torch.Tensor):
     _lib.call("clgrpo_unpad_indices", a, _stream(attn_mask))
     n_idx, max_len = total.tolist()
     return indices[:n_idx], cu, seqlens, max_len
+
+
+def thd_pack(tokens: torch.Tensor, prompt_len, response_len, align: int, pad_token: int, cp_size: int = 1,
+             cp_rank: int = 0, want_loss_mask: bool = True) -> Dict[str, object]:
+    """Packed (THD) micro-batch from per-sample lengths, in one device pass.
+
+    ``tokens`` int64 [B, S] on the device; ``prompt_len`` / ``response_len`` host sequences (or CPU
+    tensors) of B ints, from which the padded sizes are computed on the host, so no device value is
+    read back to size the outputs.  Every sequence is padded with ``pad_token`` to a multiple of
+    ``align``.  Returns a dict: ``cu_seqlens_padded`` int32 [B+1], ``seqlens`` / ``seqlens_padded`` int32
+    [B], ``indices`` int64 [total] (positions in the padded [B, max padded length] layout),
+    ``seq_indices`` / ``tokens`` / ``labels`` int64 [total / cp_size] and ``loss_mask`` int32 for this
+    context-parallel rank, ``num_loss_tokens`` (device int32 scalar), ``total_padded`` and
+    ``max_seqlen_padded`` (host ints).  Raises if the device-side sizes disagree with the host's."""
+    tokens = _dev(tokens, "tokens", torch.int64)
+    if tokens.dim() != 2:
+        raise ValueError("tokens must be [B, S]")
+    B, S = tokens.shape
+    pl = [int(x) for x in (prompt_len.tolist() if isinstance(prompt_len, torch.Tensor) else prompt_len)]
+    rl = [int(x) for x in (response_len.tolist() if isinstance(response_len, torch.Tensor) else response_len)]
+    if len(pl) != B or len(rl) != B:
+        raise ValueError(f"prompt_len / response_len must have {B} entries")
+    align, cp_size, cp_rank = int(align), int(cp_size), int(cp_rank)
+    if align <= 0 or cp_size <= 0:
+        raise ValueError("align and cp_size must be positive")
+    padded = [(p + r + align - 1) // align * align for p, r in zip(pl, rl)]
+    total, max_padded = sum(padded), max(padded)
+    dev = tokens.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    lens = torch.tensor([pl, rl], dtype=torch.int32).to(dev)
+    cu, seqlens, seqlens_padded = torch.empty(B + 1, **i32), torch.empty(B, **i32), torch.empty(B, **i32)
+    stats, status = torch.empty(3, **i32), torch.empty(1, **i32)
+    per_rank = total // cp_size
+    i64o = dict(dtype=torch.int64, device=dev)
+    indices, seq_indices = torch.empty(total, **i64o), torch.empty(per_rank, **i64o)
+    out_tokens, out_labels = torch.empty(per_rank, **i64o), torch.empty(per_rank, **i64o)
+    out_mask = torch.empty(per_rank, **i32) if want_loss_mask else None
+    a = _lib.ThdPackArgs(B, S, _ptr(tokens), _ptr(lens[0]), _ptr(lens[1]), align, cp_size, cp_rank, int(pad_token), total,
+                         _ptr(cu), _ptr(seqlens), _ptr(seqlens_padded), _ptr(stats), _ptr(status), _ptr(indices),
+                         _ptr(seq_indices), _ptr(out_tokens), _ptr(out_labels), _ptr(out_mask))
+    _lib.call("clgrpo_thd_pack", a, _stream(tokens))
+    bad = int(status.item())
+    if bad:
+        why = [m for bit, m in ((1, "padded total differs from the host's"), (2, "a sequence is longer than S"),
+                                (4, "a padded length is not a multiple of 2*cp_size")) if bad & bit]
+        raise ValueError("thd_pack: " + "; ".join(why))
+    return {"cu_seqlens_padded": cu, "seqlens": seqlens, "seqlens_padded": seqlens_padded, "indices": indices,
+            "seq_indices": seq_indices, "tokens": out_tokens, "labels": out_labels, "loss_mask": out_mask,
+            "num_loss_tokens": stats[2], "total_padded": total, "max_seqlen_padded": max_padded}
 
 
 def gather_rows(src: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:

@@ -274,6 +274,51 @@ typedef struct {
 } clgrpo_unpad_indices_args;
 int clgrpo_unpad_indices(const clgrpo_unpad_indices_args* a, void* stream);
 
+/* Packed ("THD") micro-batch for the Megatron trainer in one pass, driven by the per-sample
+ * (prompt, response) lengths.  Replaces the packed branch of get_batch
+ * (megatron_utils/train_helper.py:258-328): the O(B) Python loops that build the attention mask,
+ * pad every sequence to a multiple of align = tp*cp*2 with the eod token, unpad_input, the label
+ * roll, the loss mask placed at cu_seqlens_padded[i] + prompt and rolled, and
+ * thd_get_partitioned_indices (TransformerEngine) with the index_select calls that follow it.
+ *
+ * Row i of the padded batch holds seqlen_i = prompt_i + response_i tokens; its packed segment has
+ * padded_i = ceil(seqlen_i / align) * align tokens.  The caller passes total_padded = sum padded_i
+ * (known on the host from the same lengths); the call fails the `status` word (bit 0) if the device
+ * sum disagrees, (bit 1) if a sequence is longer than S, (bit 2) if a padded length is not a
+ * multiple of 2*cp_size.
+ * Outputs over the whole packed row (n = total_padded):
+ *   cu_seqlens_padded [B+1], seqlens [B], seqlens_padded [B]            int32
+ *   stats[0] = total_padded, stats[1] = max padded length                int32
+ *   indices [n]: position in the padded [B, max padded length] layout    int64
+ * Outputs for this context-parallel rank (m = total_padded / cp_size entries, order of seq_indices):
+ *   seq_indices [m]: positions in the packed row this rank owns (per sequence the chunks
+ *                    cp_rank and 2*cp_size-1-cp_rank of 2*cp_size equal chunks)        int64
+ *   tokens [m], labels [m] (packed row rolled left by one, wrapping)    int64
+ *   loss_mask [m] (rolled the same way)                                  int32
+ *   stats[2] = number of ones in loss_mask                               int32
+ */
+typedef struct {
+  int64_t B, S;
+  const int64_t* tokens;        /* [B,S] */
+  const int32_t* prompt_len;    /* [B] */
+  const int32_t* response_len;  /* [B] */
+  int32_t align;                /* tp*cp*2 */
+  int32_t cp_size, cp_rank;
+  int64_t pad_token;            /* tokenizer eod */
+  int64_t total_padded;
+  int32_t* cu_seqlens_padded;   /* [B+1] out */
+  int32_t* seqlens;             /* [B] out */
+  int32_t* seqlens_padded;      /* [B] out */
+  int32_t* stats;               /* [3] out */
+  int32_t* status;              /* [1] out, zero when consistent */
+  int64_t* indices;             /* [total_padded] out */
+  int64_t* seq_indices;         /* [total_padded / cp_size] out */
+  int64_t* out_tokens;          /* [total_padded / cp_size] out */
+  int64_t* out_labels;          /* [total_padded / cp_size] out */
+  int32_t* out_loss_mask;       /* [total_padded / cp_size] out, or NULL */
+} clgrpo_thd_pack_args;
+int clgrpo_thd_pack(const clgrpo_thd_pack_args* a, void* stream);
+
 typedef struct {
   const void* src;             /* gather: [n_src_rows, row_bytes]; scatter: [n_idx, row_bytes] */
   void* dst;                   /* gather: [n_idx, row_bytes];      scatter: [n_dst_rows, row_bytes] */

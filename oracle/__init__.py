@@ -23,6 +23,11 @@ of them, so none is pinned by a reference fixture):
   round-trip ``pad(unpad(x)) == x * mask``.
 * group advantages: ``numpy.mean`` / ``numpy.std`` and the Bernoulli closed
   form ``(1-k/G)/(sqrt(k/G(1-k/G))+1e-5)``.
+* the Megatron trainer's packed batch (sequence padding to tp*cp*2, unpad,
+  label roll, rolled loss mask): hand-worked cases in
+  ``tests/golden/thd_pack_cases.json``; the context-parallel index split it
+  calls from TransformerEngine is restated from the published chunk scheme and
+  is PARITY UNPINNED for more than one rank (identity for one rank).
 * vocabulary-parallel logprob / entropy (the reference's three all-reduces
   over tensor-parallel ranks): equality with the unsharded log_softmax gather
   and entropy for every way of cutting the vocabulary, and the uniform-logits

@@ -74,3 +74,74 @@ def shift_loss_mask_fsdp(loss_mask):
 def shift_loss_mask_megatron(loss_mask):
     """train_helper.py:405-413: roll left by one only."""
     return torch.roll(loss_mask, shifts=-1, dims=1)
+
+
+def thd_partitioned_indices(cu_seqlens, total_tokens, world_size, rank):
+    """Positions of a packed (THD) row that one context-parallel rank keeps.
+
+    The reference calls TransformerEngine's ``tex.thd_get_partitioned_indices``
+    (megatron_utils/train_helper.py:289-291); TransformerEngine is a third-party
+    dependency that is not vendored, so this restates its published scheme: every
+    sequence is cut into ``2 * world_size`` equal chunks and rank ``r`` keeps chunks
+    ``r`` and ``2 * world_size - 1 - r`` (load balancing under a causal mask), in
+    sequence order.  For ``world_size == 1`` this is ``arange(total_tokens)``, which
+    is all the reference's own single-rank use needs; for more ranks the parity of
+    this function with TransformerEngine is unpinned (no fixture of it exists in the
+    reference) and only its defining properties are tested.
+    """
+    out = []
+    for i in range(len(cu_seqlens) - 1):
+        start, end = int(cu_seqlens[i]), int(cu_seqlens[i + 1])
+        chunk = (end - start) // (2 * world_size)
+        for c in (rank, 2 * world_size - 1 - rank):
+            out.extend(range(start + c * chunk, start + (c + 1) * chunk))
+    assert len(out) == total_tokens // world_size
+    return torch.tensor(out, dtype=torch.int64)
+
+
+def megatron_packed_batch(tokens, prompt_token_length, response_token_length, eod, tp_size=1, cp_size=1, cp_rank=0):
+    """The packed branch of the Megatron trainer's ``get_batch`` (train_helper.py:258-328),
+    written with the same loops on CPU tensors.  Returns the dict that branch builds
+    (``packed_seq_params`` as a plain dict)."""
+    tokens = tokens.long()
+    mbs, seqlen = tokens.shape
+    align_size = tp_size * cp_size * 2
+    attn_mask = torch.zeros_like(tokens, dtype=torch.int32)
+    for i, (p, r) in enumerate(zip(prompt_token_length, response_token_length)):
+        attn_mask[i, : p + r] = 1
+    seqlens_in_batch = attn_mask.sum(dim=-1, dtype=torch.int32)
+    pad_size = (align_size - seqlens_in_batch % align_size) % align_size
+    seqlens_in_batch_padded = seqlens_in_batch + pad_size
+    width = int(seqlens_in_batch_padded.max())
+    tokens_padded = torch.full((mbs, width), eod, dtype=tokens.dtype)
+    attn_mask_for_padding = torch.zeros((mbs, width), dtype=tokens.dtype)
+    for i in range(mbs):
+        n, n_pad = int(seqlens_in_batch[i]), int(seqlens_in_batch_padded[i])
+        tokens_padded[i, :n] = tokens[i, :n]
+        attn_mask_for_padding[i, :n_pad] = 1
+    packed, indices, cu_seqlens_padded, max_seqlen_in_batch = unpad_input(tokens_padded.unsqueeze(-1),
+                                                                         attn_mask_for_padding)[:4]
+    seq_indices = thd_partitioned_indices(cu_seqlens_padded, packed.shape[0], cp_size, cp_rank)
+    tokens_rank = packed.index_select(0, seq_indices)
+    labels = torch.roll(packed, shifts=-1, dims=0)
+    labels_rank = labels.index_select(0, seq_indices)
+    loss_mask = torch.zeros_like(packed, dtype=torch.int32)
+    for i, (p, r) in enumerate(zip(prompt_token_length, response_token_length)):
+        start = int(cu_seqlens_padded[i])
+        loss_mask[start + p: start + p + r, 0] = 1
+    loss_mask = torch.roll(loss_mask, shifts=-1, dims=0)
+    loss_mask_rank = loss_mask.index_select(0, seq_indices)
+    return {
+        "all_tokens": tokens_rank.transpose(0, 1),
+        "labels": labels_rank.transpose(0, 1),
+        "packed_seq_params": {"qkv_format": "thd", "cu_seqlens_q": cu_seqlens_padded,
+                              "cu_seqlens_kv": cu_seqlens_padded, "max_seqlen_q": max_seqlen_in_batch,
+                              "max_seqlen_kv": max_seqlen_in_batch},
+        "ori_seq_len": seqlens_in_batch_padded.max(),
+        "ori_batch_size": mbs,
+        "seq_indices": seq_indices.unsqueeze(0),
+        "indices": indices,
+        "num_tokens_on_this_cp_rank": loss_mask_rank.sum(),
+        "pad_size": seqlens_in_batch_padded.max() - seqlen,
+        "loss_mask_on_this_cp_rank": loss_mask_rank,
+    }

@@ -1,0 +1,114 @@
+"""Packed (THD) micro-batches for the Megatron trainer: the device pass against the oracle's
+restatement of the reference's packed ``get_batch`` branch, bit-exact (integer work)."""
+import pytest
+import torch
+
+from oracle import indexing as oidx
+
+pytestmark = pytest.mark.gpu
+
+
+def _batch(B, S, seed, empty_row=False):
+    g = torch.Generator().manual_seed(seed)
+    p = torch.randint(1, S // 3, (B,), generator=g)
+    r = torch.randint(1, S // 2, (B,), generator=g)
+    p[0], r[0] = S // 3, S - S // 3            # one row exactly full
+    if empty_row and B > 2:
+        p[1], r[1] = 0, 0                      # an empty sample
+    tokens = torch.randint(5, 1000, (B, S), generator=g)
+    return tokens, p.tolist(), r.tolist()
+
+
+@pytest.mark.parametrize("B,S,tp,cp,rank", [
+    (5, 64, 1, 1, 0), (7, 96, 2, 1, 0), (6, 128, 1, 2, 0), (6, 128, 1, 2, 1), (9, 80, 2, 2, 1),
+    (4, 60, 4, 3, 2), (1, 32, 1, 1, 0), (300, 48, 1, 1, 0),
+])
+def test_thd_pack_matches_reference_branch(dev, B, S, tp, cp, rank):
+    from chatlearn_amd import ops
+    tokens, p, r = _batch(B, S, seed=B * 1000 + S + tp + cp, empty_row=(B == 9))
+    eod = 3
+    want = oidx.megatron_packed_batch(tokens, p, r, eod, tp_size=tp, cp_size=cp, cp_rank=rank)
+    got = ops.thd_pack(tokens.to(dev), p, r, align=tp * cp * 2, pad_token=eod, cp_size=cp, cp_rank=rank)
+    cu = want["packed_seq_params"]["cu_seqlens_q"]
+    assert torch.equal(got["cu_seqlens_padded"].cpu(), cu)
+    assert got["max_seqlen_padded"] == want["packed_seq_params"]["max_seqlen_q"] == int(want["ori_seq_len"])
+    assert got["total_padded"] == int(cu[-1])
+    assert torch.equal(got["indices"].cpu(), want["indices"])
+    assert torch.equal(got["seq_indices"].cpu(), want["seq_indices"][0])
+    assert torch.equal(got["tokens"].cpu(), want["all_tokens"][0])
+    assert torch.equal(got["labels"].cpu(), want["labels"][0])
+    assert torch.equal(got["loss_mask"].cpu(), want["loss_mask_on_this_cp_rank"][:, 0])
+    assert int(got["num_loss_tokens"]) == int(want["num_tokens_on_this_cp_rank"])
+    assert torch.equal(got["seqlens"].cpu(), torch.tensor([a + b for a, b in zip(p, r)], dtype=torch.int32))
+
+
+def test_ranks_partition_the_packed_row(dev):
+    """Defining property of the context-parallel split: the ranks' shares are disjoint, cover the row,
+    and per sequence a rank holds chunks r and 2*cp-1-r of 2*cp equal chunks."""
+    from chatlearn_amd import ops
+    tokens, p, r = _batch(6, 120, seed=11)
+    cp = 3
+    parts = [ops.thd_pack(tokens.to(dev), p, r, align=2 * cp, pad_token=0, cp_size=cp, cp_rank=k) for k in range(cp)]
+    every = torch.cat([x["seq_indices"] for x in parts]).cpu()
+    total = parts[0]["total_padded"]
+    assert torch.equal(every.sort().values, torch.arange(total))
+    cu = parts[0]["cu_seqlens_padded"].cpu().tolist()
+    for k, part in enumerate(parts):
+        idx = part["seq_indices"].cpu()
+        for i in range(6):
+            chunk = (cu[i + 1] - cu[i]) // (2 * cp)
+            mine = idx[(idx >= cu[i]) & (idx < cu[i + 1])] - cu[i]
+            assert sorted(set((mine // chunk).tolist())) == sorted({k, 2 * cp - 1 - k})
+    assert sum(int(x["num_loss_tokens"]) for x in parts) == sum(r)
+
+
+def test_get_batch_packed_keys_and_training_fields(dev):
+    from chatlearn_amd.algorithm.grpo_utils.megatron_utils.train_helper import get_batch_packed
+    tokens, p, r = _batch(5, 64, seed=3)
+    data_b = {"all_tokens": tokens, "prompt_token_length": p, "response_token_length": r,
+              "ref_logprobs": torch.zeros(5, 64, dtype=torch.float64), "old_logprobs": torch.zeros(5, 64),
+              "advantages": [0.5] * 5}
+    out = get_batch_packed(data_b, True, eod=7, tp_size=2, device=dev)
+    want = oidx.megatron_packed_batch(tokens, p, r, 7, tp_size=2)
+    for key in ("all_tokens", "labels", "seq_indices", "indices"):
+        assert torch.equal(out[key].cpu(), want[key]), key
+    assert out["ori_batch_size"] == 5 and out["ori_seq_len"] == int(want["ori_seq_len"])
+    assert out["pad_size"] == int(want["pad_size"])
+    assert int(out["num_tokens_on_this_cp_rank"]) == int(want["num_tokens_on_this_cp_rank"])
+    assert out["packed_seq_params"].qkv_format == "thd"
+    assert torch.equal(out["packed_seq_params"].cu_seqlens_q.cpu(), want["packed_seq_params"]["cu_seqlens_q"])
+    # the [mbs, seq_length] training mask: ones on the response, rolled left by one (train_helper.py:405-413)
+    lm = torch.zeros(5, 64, dtype=torch.int32)
+    for i in range(5):
+        lm[i, p[i]: p[i] + r[i]] = 1
+    assert torch.equal(out["all_token_loss_mask"].cpu(), torch.roll(lm, shifts=-1, dims=1))
+    assert out["ref_logprobs"].dtype == torch.float32 and out["old_logprobs"].is_cuda
+
+
+def test_thd_pack_rejects_inconsistent_input(dev):
+    from chatlearn_amd import ops
+    tokens, p, r = _batch(4, 32, seed=1)
+    p[2], r[2] = 30, 10                        # longer than the row
+    with pytest.raises(ValueError, match="longer than S"):
+        ops.thd_pack(tokens.to(dev), p, r, align=2, pad_token=0)
+    with pytest.raises(ValueError):
+        ops.thd_pack(tokens.to(dev), p[:3], r[:3], align=2, pad_token=0)
+
+
+def test_thd_pack_against_hand_worked_cases(dev):
+    import json
+    import os
+    from chatlearn_amd import ops
+    with open(os.path.join(os.path.dirname(__file__), "golden", "thd_pack_cases.json")) as f:
+        gold = json.load(f)
+    tokens = torch.tensor(gold["tokens"]).to(dev)
+    for c in gold["cases"]:
+        got = ops.thd_pack(tokens, gold["prompt"], gold["response"], align=c["tp"] * c["cp"] * 2, pad_token=gold["eod"],
+                           cp_size=c["cp"], cp_rank=c["rank"])
+        assert got["cu_seqlens_padded"].tolist() == c["cu_seqlens_padded"]
+        assert got["indices"].tolist() == c["indices"]
+        assert got["seq_indices"].tolist() == c["seq_indices"]
+        assert got["tokens"].tolist() == c["all_tokens"]
+        assert got["labels"].tolist() == c["labels"]
+        assert got["loss_mask"].tolist() == c["loss_mask"]
+        assert int(got["num_loss_tokens"]) == c["num_tokens"]

@@ -313,3 +313,22 @@ def test_vocab_parallel_oracle_equals_unsharded_for_any_split(n):
     assert torch.allclose(ovp.vocab_parallel_entropy(u), torch.full((3,), math.log(24.0)))
     assert torch.allclose(ovp.vocab_parallel_logprob(u, torch.tensor([0, 11, 23]), ranges),
                           torch.full((3,), -math.log(24.0)))
+
+
+def test_megatron_packed_batch_oracle_against_hand_worked_cases():
+    import json
+    import os
+    from oracle import indexing as oidx
+    with open(os.path.join(os.path.dirname(__file__), "golden", "thd_pack_cases.json")) as f:
+        gold = json.load(f)
+    tokens = torch.tensor(gold["tokens"])
+    for c in gold["cases"]:
+        out = oidx.megatron_packed_batch(tokens, gold["prompt"], gold["response"], gold["eod"], tp_size=c["tp"],
+                                         cp_size=c["cp"], cp_rank=c["rank"])
+        assert out["packed_seq_params"]["cu_seqlens_q"].tolist() == c["cu_seqlens_padded"]
+        assert out["indices"].tolist() == c["indices"]
+        assert out["seq_indices"][0].tolist() == c["seq_indices"]
+        assert out["all_tokens"][0].tolist() == c["all_tokens"]
+        assert out["labels"][0].tolist() == c["labels"]
+        assert out["loss_mask_on_this_cp_rank"][:, 0].tolist() == c["loss_mask"]
+        assert int(out["num_tokens_on_this_cp_rank"]) == c["num_tokens"] and int(out["pad_size"]) == c["pad_size"]
