@@ -223,6 +223,7 @@ struct GemmParams {
   int accumulate;
   int k_split;        // > 1: work item = (tile, K range); fp32 partial tiles go to `partial`
   int k_per_split;    // K extent of one range, a multiple of the slab
+  int n_walk;         // > 0: workgroups walk runs of m tiles (see gemm_nt_kernel); needs k_split == 1
   float* partial;     // [k_split][M][N] fp32, row stride N
 };
 
@@ -230,38 +231,15 @@ template <typename OutT> __device__ __forceinline__ OutT cvt_out(float v);
 template <> __device__ __forceinline__ float cvt_out<float>(float v) { return v; }
 template <> __device__ __forceinline__ __bf16 cvt_out<__bf16>(float v) { return (__bf16)v; }
 
+// Output tile (mt, nt) from the accumulators: C (+)= acc, or the fp32 partial of K range `ks`.
 template <typename T, typename OutT>
-__global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
+__device__ __forceinline__ void gemm_store_tile(const GemmParams& p, f32x16 (&acc)[HeadTile<T>::MI][HeadTile<T>::NI],
+                                                int m0, int n0, int a_rows, int b_rows, int ks) {
   using Tile = HeadTile<T>;
   constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
-  extern __shared__ __align__(16) char lds[];
-
-  int item = xcd_remap(blockIdx.x, gridDim.x);
-  if (item >= p.n_mt * p.n_nt * p.k_split) return;
-  const int ks = item / (p.n_mt * p.n_nt);
-  item -= ks * (p.n_mt * p.n_nt);
-  int mt, nt;
-  grouped_tile(item, p.n_mt, p.n_nt, 8, mt, nt);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave % 2, wn = wave / 2;
-  const int m0 = mt * 256, n0 = nt * 256;
-  const int a_rows = (p.M - m0) < 256 ? (p.M - m0) : 256;
-  const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
-  const int k0 = ks * p.k_per_split;
-  const int k_len = (p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split;
-
-  f32x16 acc[MI][NI];
-#pragma unroll
-  for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
-
-  Tile::run(acc, static_cast<const T*>(p.A) + (int64_t)m0 * p.lda + k0, p.lda, a_rows,
-            static_cast<const T*>(p.B) + (int64_t)n0 * p.ldb + k0, p.ldb, b_rows, k_len, lds);
-
   if (p.k_split > 1) {
     float* P = p.partial + (int64_t)ks * p.M * p.N;
 #pragma unroll
@@ -278,7 +256,6 @@ __global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
     }
     return;
   }
-
   OutT* C = static_cast<OutT*>(p.C);
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
@@ -297,6 +274,69 @@ __global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
         }
       }
   }
+}
+
+// Work item = (walk, n tile) when n_walk > 0: the workgroup walks a contiguous run of m tiles
+// for one n tile, so B rows stay the same and the K loops stream into each other (the next
+// tile's first slabs are requested while the current tile finishes and is stored).  Otherwise
+// work item = (K range, m tile, n tile), one K loop per workgroup.
+template <typename T, typename OutT>
+__global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
+  using Tile = HeadTile<T>;
+  constexpr int MI = Tile::MI, NI = Tile::NI;
+  extern __shared__ __align__(16) char lds[];
+
+  int item = xcd_remap(blockIdx.x, gridDim.x);
+  f32x16 acc[MI][NI];
+  if (p.n_walk > 0) {
+    if (item >= p.n_walk * p.n_nt) return;
+    int walk, nt;
+    grouped_tile(item, p.n_walk, p.n_nt, 4, walk, nt);
+    const int mt_begin = (int)((int64_t)walk * p.n_mt / p.n_walk);
+    const int mt_end = (int)((int64_t)(walk + 1) * p.n_mt / p.n_walk);
+    const int n0 = nt * 256;
+    const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
+    const T* B = static_cast<const T*>(p.B) + (int64_t)n0 * p.ldb;
+    typename Tile::Stream st;
+    for (int mt = mt_begin; mt < mt_end; ++mt) {
+      const int m0 = mt * 256;
+      const int a_rows = (p.M - m0) < 256 ? (p.M - m0) : 256;
+      const int m1 = m0 + 256;
+      const int next_rows = (p.M - m1) < 256 ? (p.M - m1) : 256;
+      const T* A = static_cast<const T*>(p.A) + (int64_t)m0 * p.lda;
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+      Tile::run(acc, A, p.lda, a_rows, B, p.ldb, b_rows, p.K, lds, st,
+                (mt + 1 < mt_end) ? A + (int64_t)256 * p.lda : nullptr, next_rows, true);
+      gemm_store_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows, 0);
+    }
+    return;
+  }
+
+  if (item >= p.n_mt * p.n_nt * p.k_split) return;
+  const int ks = item / (p.n_mt * p.n_nt);
+  item -= ks * (p.n_mt * p.n_nt);
+  int mt, nt;
+  grouped_tile(item, p.n_mt, p.n_nt, 8, mt, nt);
+  const int m0 = mt * 256, n0 = nt * 256;
+  const int a_rows = (p.M - m0) < 256 ? (p.M - m0) : 256;
+  const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
+  const int k0 = ks * p.k_per_split;
+  const int k_len = (p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split;
+#pragma unroll
+  for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+
+  Tile::run(acc, static_cast<const T*>(p.A) + (int64_t)m0 * p.lda + k0, p.lda, a_rows,
+            static_cast<const T*>(p.B) + (int64_t)n0 * p.ldb + k0, p.ldb, b_rows, k_len, lds);
+  gemm_store_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows, ks);
 }
 
 // C[m][n] (+)= sum over splits of partial[s][m][n]
@@ -408,7 +448,14 @@ static int launch_gemm(const void* A, int64_t lda, int M, const void* B, int64_t
   g.k_split = partial ? pick_k_split(g.n_mt * g.n_nt, M, N, K, slab, partial_bytes) : 1;
   g.k_per_split = g.k_split > 1 ? (int)round_up64((K + g.k_split - 1) / g.k_split, slab) : K;
   g.partial = partial;
-  int grid = (g.n_mt * g.n_nt * g.k_split + 7) / 8 * 8;
+  // Many more tiles than CUs and no K split: let 256 workgroups walk runs of m tiles instead of
+  // launching one workgroup per tile.
+  g.n_walk = 0;
+  if (g.k_split == 1 && g.n_nt <= 256 && g.n_mt * g.n_nt >= 4 * 256 && K >= 2 * slab) {
+    g.n_walk = 256 / g.n_nt;
+    if (g.n_walk > g.n_mt) g.n_walk = g.n_mt;
+  }
+  int grid = ((g.n_walk > 0 ? g.n_walk * g.n_nt : g.n_mt * g.n_nt * g.k_split) + 7) / 8 * 8;
   hipLaunchKernelGGL((gemm_nt_kernel<T, OutT>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, g);
   int rc = check_launch("gemm_nt_kernel");
   if (rc || g.k_split == 1) return rc;

@@ -135,3 +135,26 @@ def test_argument_errors(dev):
     w = torch.randn(10, 64, device=dev)
     lp, *_ = ops.lmhead_forward(h, w, torch.tensor([0, 9, 10, -1], device=dev))
     assert torch.isfinite(lp[:2]).all() and torch.isnan(lp[2:]).all()
+
+
+def test_backward_weight_gradient_with_walking_workgroups(dev):
+    """A weight-gradient GEMM with many more 256 x 256 tiles than CUs runs with workgroups that walk
+    runs of tiles (consecutive K loops streaming into each other); ragged V and T edges included."""
+    from chatlearn_amd import ops
+    T, H, V = 200, 4096, 16400
+    hidden, weight, labels = _inputs(T, H, V, torch.bfloat16, seed=9, w_std=0.02)
+    g = torch.Generator().manual_seed(6)
+    g_lp = torch.randn(T, generator=g)
+    g_ent = torch.randn(T, generator=g) * 0.1
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld, 1.0)
+    dh, dw = ops.lmhead_backward(hd, wd, ld, lse, ent, g_lp.to(dev), g_ent.to(dev), 1.0)
+    rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, g_lp, g_ent, 1.0)
+    assert_close_rel(dh, rdh, 1e-2, "dhidden")
+    assert_close_rel(dw, rdw, 1e-2, "dweight")
+    # accumulate into an existing fp32 buffer
+    base = torch.randn(V, H, generator=g)
+    acc = base.clone().to(dev)
+    ops.lmhead_backward(hd, wd, ld, lse, ent, g_lp.to(dev), g_ent.to(dev), 1.0, need_dhidden=False, dweight=acc,
+                        accumulate_dweight=True)
+    assert_close_rel(acc - base.to(dev), rdw, 1e-2, "accumulated dweight")
