@@ -33,10 +33,19 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kRowBytes = 128;    // K-slab bytes per tile row
 constexpr int kChunksPerRow = 8;  // 16-byte chunks per slab row
+constexpr int kBlockRows = 256;   // rows per block of a K-blocked operand
 
 template <typename T> struct Elem;
 template <> struct Elem<__bf16> { static constexpr int kSlabK = 64; };
 template <> struct Elem<float> { static constexpr int kSlabK = 32; };
+
+// Element (row, k) of a K-blocked operand with `n_kslab` slabs per row: blocks of 256 rows, each
+// block holding its slabs one after another, each slab 256 rows of 128 bytes.
+template <typename T>
+__host__ __device__ __forceinline__ int64_t blocked_index(int64_t row, int64_t k, int64_t n_kslab) {
+  constexpr int E = kRowBytes / (int)sizeof(T);
+  return (((row / kBlockRows) * n_kslab + k / E) * kBlockRows + (row % kBlockRows)) * E + (k % E);
+}
 
 // One 32-byte-of-K step for a 32x32 block: a and b each hold 16 bytes per lane.
 template <typename T>
@@ -87,36 +96,62 @@ struct GemmTile {
     bool loaded = false;
   };
 
+  // Where an operand's tile lives in memory: `rows` valid rows starting at `base`, consecutive
+  // rows `row_bytes` apart, consecutive 128-byte K slabs of a row `slab_bytes` apart.
+  //   row-major [rows][ld]:                  row_bytes = ld * sizeof(T), slab_bytes = 128
+  //   K-blocked [row block][K slab][256][128 B]: row_bytes = 128, slab_bytes = 256 * 128 (one
+  //   contiguous 32 KB piece per tile and slab)
+  struct Operand {
+    const T* base;
+    int row_bytes;
+    int slab_bytes;
+    int rows;
+    __device__ static __forceinline__ Operand row_major(const T* base, int64_t ld, int rows) {
+      return Operand{base, (int)(ld * (int64_t)sizeof(T)), kRowBytes, rows};
+    }
+    __device__ static __forceinline__ Operand blocked(const T* block_base, int rows) {
+      return Operand{block_base, kRowBytes, kBlockRows * kRowBytes, rows};
+    }
+  };
+
   // Per-thread constants of the global -> LDS loads of one operand pair.
   struct Loader {
-    __amdgpu_buffer_rsrc_t a_rsrc, b_rsrc;
+    const char* a_ptr;
+    const char* b_ptr;
+    int a_bytes, b_bytes;     // bytes the valid rows span from the tile base at slab 0
+    int a_shrink, b_shrink;   // by how much that span shrinks per slab step (row-major: one slab; blocked: 0)
+    int a_slab, b_slab;
     int a_voff, b_voff, a_pass, b_pass, dma_off;
   };
 
   typedef __attribute__((address_space(3))) char lds_char;
 
-  // Loads go through range-checked buffer descriptors that cover exactly the a_rows / b_rows
-  // valid rows, so rows past them read as zero and nothing outside the operands is touched.
-  // The row part of an address always travels in the per-lane offset (the part the hardware
-  // range check is guaranteed to see); only the in-row K offset rides in the scalar offset.
-  __device__ static __forceinline__ Loader make_loader(const T* a_base, int64_t lda, int a_rows,
-                                                       const T* b_base, int64_t ldb, int b_rows) {
+  // Loads go through range-checked buffer descriptors that cover exactly the valid rows, so rows
+  // past them read as zero and nothing outside the operands is touched.  The hardware checks the
+  // sum of the per-lane and the scalar offset against the descriptor's size, so the K-slab offset
+  // travels in the descriptor's base address instead (a few scalar instructions per slab) and the
+  // size is what is left of the valid rows from there.
+  __device__ static __forceinline__ Loader make_loader(const Operand& a, const Operand& b) {
     const int tid = threadIdx.x;
     const int ld_row = tid >> 3;
     const int ld_chunk = tid & 7;
-    const int lda_b = (int)(lda * (int64_t)sizeof(T));
-    const int ldb_b = (int)(ldb * (int64_t)sizeof(T));
     Loader L;
-    L.a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_base), 0, a_rows * lda_b, 0x00020000);
-    L.b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(b_base), 0, b_rows * ldb_b, 0x00020000);
+    L.a_ptr = reinterpret_cast<const char*>(a.base);
+    L.b_ptr = reinterpret_cast<const char*>(b.base);
+    L.a_bytes = a.rows * a.row_bytes;
+    L.b_bytes = b.rows * b.row_bytes;
+    L.a_shrink = a.slab_bytes == kRowBytes ? kRowBytes : 0;
+    L.b_shrink = b.slab_bytes == kRowBytes ? kRowBytes : 0;
+    L.a_slab = a.slab_bytes;
+    L.b_slab = b.slab_bytes;
     // A wave's load instruction fills 1 KB of LDS in lane order: 8 rows x 8 chunks of 16 bytes.
     // The lane that lands on (row, slot) fetches K-chunk slot ^ swz(row), so a fragment read of
     // K-chunk q goes to slot q ^ swz(row).
     const int ld_swz = (ld_row & 7) ^ ((ld_row >> 3) & 1);
-    L.a_voff = ld_row * lda_b + ((ld_chunk ^ ld_swz) * 16);
-    L.b_voff = ld_row * ldb_b + ((ld_chunk ^ ld_swz) * 16);
-    L.a_pass = kRowsPerPass * lda_b;
-    L.b_pass = kRowsPerPass * ldb_b;
+    L.a_voff = ld_row * a.row_bytes + ((ld_chunk ^ ld_swz) * 16);
+    L.b_voff = ld_row * b.row_bytes + ((ld_chunk ^ ld_swz) * 16);
+    L.a_pass = kRowsPerPass * a.row_bytes;
+    L.b_pass = kRowsPerPass * b.row_bytes;
     L.dma_off = __builtin_amdgcn_readfirstlane(tid >> 6) * 8 * kRowBytes;   // this wave's 8 rows within a pass
     return L;
   }
@@ -124,42 +159,45 @@ struct GemmTile {
   // global -> LDS without passing registers; completion must be awaited (wait_loads) before the
   // workgroup barrier that publishes the stage.
   __device__ static __forceinline__ void dma_slab(const Loader& L, char* stage, int slab) {
-    const int koff = slab * kRowBytes;
     lds_char* dst = (lds_char*)(stage) + L.dma_off;
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(L.a_ptr + (int64_t)slab * L.a_slab), 0, L.a_bytes - slab * L.a_shrink, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(L.b_ptr + (int64_t)slab * L.b_slab), 0, L.b_bytes - slab * L.b_shrink, 0x00020000);
 #pragma unroll
     for (int p = 0; p < kPassA; ++p)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(L.a_rsrc, dst + p * kRowsPerPass * kRowBytes, 16,
-                                               L.a_voff + p * L.a_pass, koff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, dst + p * kRowsPerPass * kRowBytes, 16,
+                                               L.a_voff + p * L.a_pass, 0, 0, 0);
 #pragma unroll
     for (int p = 0; p < kPassB; ++p)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(L.b_rsrc, dst + (BM + p * kRowsPerPass) * kRowBytes, 16,
-                                               L.b_voff + p * L.b_pass, koff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, dst + (BM + p * kRowsPerPass) * kRowBytes, 16,
+                                               L.b_voff + p * L.b_pass, 0, 0, 0);
   }
 
   // A workgroup barrier does not wait for loads whose destination is LDS: wait for this wave's
   // outstanding ones explicitly (s_waitcnt vmcnt(0), the other counters left alone).
   __device__ static __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-  // acc[mi][ni] must be zeroed by the caller.  a_base/b_base point at row 0 of the tile (K offset
-  // 0).  K must be a multiple of kSlabK and the rows 16-byte aligned.  With a_next != nullptr the
-  // last two slab periods request the first two slabs of the next K loop (A rows from a_next, same
-  // B), and LDS stays in use on return; otherwise, with release_lds, all loads have landed and
-  // every wave is past its last fragment read on return.
-  __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const T* a_base, int64_t lda,
-                                             int a_rows, const T* b_base, int64_t ldb, int b_rows,
-                                             int K, char* lds, Stream& st, const T* a_next,
-                                             int a_next_rows, bool release_lds) {
+  // acc[mi][ni] must be zeroed by the caller.  `a` / `b` describe the tile's rows from K offset 0;
+  // K must be a multiple of kSlabK and every row 16-byte aligned.  With a_next != nullptr the last
+  // two slab periods request the first two slabs of the next K loop (A rows from a_next with
+  // a_next_rows valid rows, same layout as `a`; same B), and LDS stays in use on return; otherwise,
+  // with release_lds, all loads have landed and every wave is past its last fragment read on return.
+  __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const Operand& a, const Operand& b, int K,
+                                             char* lds, Stream& st, const T* a_next, int a_next_rows,
+                                             bool release_lds) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave % WAVES_M;
     const int wn = wave / WAVES_M;
-    const Loader L = make_loader(a_base, lda, a_rows, b_base, ldb, b_rows);
+    const Loader L = make_loader(a, b);
     const int nslab = K / kSlabK;
     const bool stream_on = a_next != nullptr && nslab >= 2;
     Loader LN = L;
-    if (stream_on)
-      LN.a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_next), 0,
-                                                    a_next_rows * (int)(lda * (int64_t)sizeof(T)), 0x00020000);
+    if (stream_on) {
+      LN.a_ptr = reinterpret_cast<const char*>(a_next);
+      LN.a_bytes = a_next_rows * a.row_bytes;
+    }
 
     const int fr_swz = (lane & 7) ^ ((lane >> 3) & 1);
     int xk[4];
@@ -253,11 +291,10 @@ struct GemmTile {
   }
 
   // Single K loop: nothing carried over, LDS free on return.
-  __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const T* a_base, int64_t lda,
-                                             int a_rows, const T* b_base, int64_t ldb, int b_rows,
-                                             int K, char* lds) {
+  __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const Operand& a, const Operand& b, int K,
+                                             char* lds) {
     Stream st;
-    run(acc, a_base, lda, a_rows, b_base, ldb, b_rows, K, lds, st, nullptr, 0, true);
+    run(acc, a, b, K, lds, st, nullptr, 0, true);
   }
 };
 

@@ -48,8 +48,8 @@ struct DzParams {
   int ldv;      // dz row stride = V rounded up to 64
   int n_tb, n_vt;
   float c, inv_temperature;
-  void* dz;     // [Tc][ldv]
-  void* dzT;    // [V][ldt]
+  void* dz;     // Tc x ldv, K-blocked (see blocked_index)
+  void* dzT;    // V x ldt, K-blocked
 };
 
 template <typename T>
@@ -102,7 +102,8 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_dz_kernel(DzParams p) {
     for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
-  if (block_live) Tile::run(acc, weight, p.H, a_rows, hidden, p.H, b_rows, p.H, lds);
+  if (block_live)
+    Tile::run(acc, Tile::Operand::row_major(weight, p.H, a_rows), Tile::Operand::row_major(hidden, p.H, b_rows), p.H, lds);
 
   T* dz = static_cast<T*>(p.dz);
   T* dzT = static_cast<T*>(p.dzT);
@@ -131,12 +132,13 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_dz_kernel(DzParams p) {
         const int v_idx = v0 + row0;
         if (tl[ni] < p.Tc && v_idx < p.ldv) {
           typedef typename Pack4<T>::type P4;
-          *reinterpret_cast<P4*>(dz + (int64_t)tl[ni] * p.ldv + v_idx) = Pack4<T>::make(d[0], d[1], d[2], d[3]);
+          *reinterpret_cast<P4*>(dz + blocked_index<T>(tl[ni], v_idx, p.ldv / Tile::kSlabK)) =
+              Pack4<T>::make(d[0], d[1], d[2], d[3]);
         }
         if (tl[ni] < p.ldt) {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
-            if (v_idx + j < p.V) dzT[(int64_t)(v_idx + j) * p.ldt + tl[ni]] = (T)d[j];
+            if (v_idx + j < p.V) dzT[blocked_index<T>(v_idx + j, tl[ni], p.ldt / Tile::kSlabK)] = (T)d[j];
         }
       }
     }
@@ -146,10 +148,12 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_dz_kernel(DzParams p) {
 // d(logits) from stored logits, in place, plus its transpose.  One 64 x 64 (token x vocabulary)
 // tile per workgroup: read z (16 bytes per lane along the vocabulary), form dz with the per-token
 // coefficients, write it back over z, and turn the tile through LDS so dzT[vocab][token] is also
-// written in 16-byte pieces.  HBM-bound: reads 1x, writes 2x the chunk.
+// written in 16-byte pieces.  Both are K-blocked operands of the GEMMs that follow, so a tile's
+// 64 rows of 128 bytes are one contiguous 8 KB run on either side.  HBM-bound: reads 1x, writes
+// 2x the chunk.
 struct DzFromZParams {
-  void* z;            // [Tc][ldv] in: raw logits, out: dz
-  void* dzT;          // [V][ldt]
+  void* z;            // Tc x ldv, K-blocked; in: raw logits, out: dz
+  void* dzT;          // V x ldt, K-blocked
   const int64_t* labels;
   int64_t label_offset;
   const float* lse;
@@ -163,6 +167,7 @@ struct DzFromZParams {
 template <typename T>
 __global__ __launch_bounds__(256) void dz_from_z_kernel(DzFromZParams p) {
   constexpr int VEC = 16 / (int)sizeof(T);       // elements per 16-byte access
+  constexpr int kE = kRowBytes / (int)sizeof(T); // elements per K slab of a blocked operand
   constexpr int CPR = 64 / VEC;                  // accesses per 64-wide tile row
   constexpr int RPP = 256 / CPR;                 // tile rows covered per pass
   __shared__ T tile[64][64 + VEC];               // [vocab][token], padded rows
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(256) void dz_from_z_kernel(DzFromZParams p) {
         const float lse2 = lse * kLog2e;
         const float ent = p.g_ent ? p.entropy[t] : 0.f;
         const int64_t lab = p.labels[t] - p.label_offset;
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(z + (int64_t)t * p.ldv + v);
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(z + blocked_index<T>(t, v, p.ldv / kE));
         const T* in = reinterpret_cast<const T*>(&raw);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
@@ -198,7 +203,7 @@ __global__ __launch_bounds__(256) void dz_from_z_kernel(DzFromZParams p) {
           vals[j] = (T)d;
         }
       }
-      *reinterpret_cast<u32x4*>(z + (int64_t)t * p.ldv + v) = *reinterpret_cast<const u32x4*>(vals);
+      *reinterpret_cast<u32x4*>(z + blocked_index<T>(t, v, p.ldv / kE)) = *reinterpret_cast<const u32x4*>(vals);
     }
 #pragma unroll
     for (int j = 0; j < VEC; ++j) tile[c * VEC + j][rr] = vals[j];
@@ -208,16 +213,16 @@ __global__ __launch_bounds__(256) void dz_from_z_kernel(DzFromZParams p) {
     const int v = v0 + rr;
     const int t = t0 + c * VEC;
     if (v < p.V && t < p.ldt)
-      *reinterpret_cast<u32x4*>(dzT + (int64_t)v * p.ldt + t) = *reinterpret_cast<const u32x4*>(&tile[rr][c * VEC]);
+      *reinterpret_cast<u32x4*>(dzT + blocked_index<T>(v, t, p.ldt / kE)) = *reinterpret_cast<const u32x4*>(&tile[rr][c * VEC]);
   }
 }
 
-// C[m][n] (+)= alpha * sum_k A[m][k] B[n][k];  C row-major with leading dimension ldc.
+// C[m][n] (+)= sum_k A[m][k] B[n][k];  C row-major with leading dimension ldc, A and B K-blocked.
 struct GemmParams {
-  const void* A;
-  const void* B;
+  const void* A;      // M x K, K-blocked with a_kslabs slabs per row block
+  const void* B;      // N x K, K-blocked with b_kslabs slabs per row block
   void* C;
-  int64_t lda, ldb, ldc;
+  int64_t a_kslabs, b_kslabs, ldc;
   int M, N, K;
   int n_mt, n_nt;
   int accumulate;
@@ -296,22 +301,23 @@ __global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
     const int mt_end = (int)((int64_t)(walk + 1) * p.n_mt / p.n_walk);
     const int n0 = nt * 256;
     const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
-    const T* B = static_cast<const T*>(p.B) + (int64_t)n0 * p.ldb;
+    constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;   // elements of one block's slab
+    const T* B = static_cast<const T*>(p.B) + (int64_t)nt * p.b_kslabs * kSlabElems;
     typename Tile::Stream st;
     for (int mt = mt_begin; mt < mt_end; ++mt) {
       const int m0 = mt * 256;
       const int a_rows = (p.M - m0) < 256 ? (p.M - m0) : 256;
       const int m1 = m0 + 256;
       const int next_rows = (p.M - m1) < 256 ? (p.M - m1) : 256;
-      const T* A = static_cast<const T*>(p.A) + (int64_t)m0 * p.lda;
+      const T* A = static_cast<const T*>(p.A) + (int64_t)mt * p.a_kslabs * kSlabElems;
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
-      Tile::run(acc, A, p.lda, a_rows, B, p.ldb, b_rows, p.K, lds, st,
-                (mt + 1 < mt_end) ? A + (int64_t)256 * p.lda : nullptr, next_rows, true);
+      Tile::run(acc, Tile::Operand::blocked(A, a_rows), Tile::Operand::blocked(B, b_rows), p.K, lds, st,
+                (mt + 1 < mt_end) ? A + p.a_kslabs * kSlabElems : nullptr, next_rows, true);
       gemm_store_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows, 0);
     }
     return;
@@ -334,8 +340,11 @@ __global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
-  Tile::run(acc, static_cast<const T*>(p.A) + (int64_t)m0 * p.lda + k0, p.lda, a_rows,
-            static_cast<const T*>(p.B) + (int64_t)n0 * p.ldb + k0, p.ldb, b_rows, k_len, lds);
+  constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;
+  const int64_t s0 = k0 / Tile::kSlabK;   // first slab of this K range
+  Tile::run(acc, Tile::Operand::blocked(static_cast<const T*>(p.A) + ((int64_t)mt * p.a_kslabs + s0) * kSlabElems, a_rows),
+            Tile::Operand::blocked(static_cast<const T*>(p.B) + ((int64_t)nt * p.b_kslabs + s0) * kSlabElems, b_rows),
+            k_len, lds);
   gemm_store_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows, ks);
 }
 
@@ -353,11 +362,13 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, int k_sp
   }
 }
 
-// dst[c][r] = src[r][c] for r < R, c < C; dst[c][r] = 0 for R <= r < ld_dst.  64x64 tiles.
+// dst(c, r) = src[r][c] for r < R, c < C and 0 for R <= r < ld_dst, where dst is the K-blocked
+// operand with C rows and ld_dst K elements (see blocked_index).  64x64 tiles.
 template <typename T>
-__global__ __launch_bounds__(256) void transpose_pad_kernel(const T* __restrict__ src, int64_t ld_src,
-                                                            T* __restrict__ dst, int64_t ld_dst, int R, int C) {
+__global__ __launch_bounds__(256) void transpose_block_kernel(const T* __restrict__ src, int64_t ld_src,
+                                                              T* __restrict__ dst, int64_t ld_dst, int R, int C) {
   __shared__ T tile[64][65];
+  constexpr int kE = kRowBytes / (int)sizeof(T);
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   for (int i = ty; i < 64; i += 4) {
@@ -367,14 +378,14 @@ __global__ __launch_bounds__(256) void transpose_pad_kernel(const T* __restrict_
   __syncthreads();
   for (int i = ty; i < 64; i += 4) {
     const int c = c0 + i, r = r0 + tx;
-    if (c < C && r < ld_dst) dst[(int64_t)c * ld_dst + r] = tile[tx][i];
+    if (c < C && r < ld_dst) dst[blocked_index<T>(c, r, ld_dst / kE)] = tile[tx][i];
   }
 }
 
 struct BwdPlan {
-  int64_t ldv;        // dz / WT row stride
+  int64_t ldv;        // K extent of dz / WT (V rounded up to 64)
   int64_t chunk;      // tokens per chunk (multiple of 256 unless >= T)
-  int64_t ldt;        // dzT / hidT row stride for a full chunk
+  int64_t ldt;        // K extent of dzT / hidT for a full chunk (tokens rounded up to 64)
   size_t off_wt, off_hidt, off_dz, off_dzt, off_part, part_bytes, total;
 };
 
@@ -386,10 +397,12 @@ static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chun
   pl.chunk = chunk;
   pl.ldt = round_up64(chunk, 64);
   size_t off = 0;
-  pl.off_wt = off;   off += align_up((size_t)H * pl.ldv * es, 256);
-  pl.off_hidt = off; off += align_up((size_t)H * pl.ldt * es, 256);
-  pl.off_dz = off;   off += saved ? 0 : align_up((size_t)chunk * pl.ldv * es, 256);
-  pl.off_dzt = off;  off += align_up((size_t)V * pl.ldt * es, 256);
+  // K-blocked operands: whole blocks of 256 rows
+  const size_t Hb = (size_t)round_up64(H, 256), Cb = (size_t)round_up64(chunk, 256), Vb = (size_t)round_up64(V, 256);
+  pl.off_wt = off;   off += align_up(Hb * pl.ldv * es, 256);
+  pl.off_hidt = off; off += align_up(Hb * pl.ldt * es, 256);
+  pl.off_dz = off;   off += saved ? 0 : align_up(Cb * pl.ldv * es, 256);
+  pl.off_dzt = off;  off += align_up(Vb * pl.ldt * es, 256);
   pl.part_bytes = align_up((size_t)4 * chunk * H * sizeof(float), 256);   // split-K partials of dhidden
   pl.off_part = off; off += pl.part_bytes;
   pl.total = off;
@@ -429,7 +442,7 @@ static int pick_k_split(int tiles, int M, int N, int K, int slab, size_t partial
 }
 
 template <typename T, typename OutT>
-static int launch_gemm(const void* A, int64_t lda, int M, const void* B, int64_t ldb, int N, int K, void* C,
+static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, int64_t b_kslabs, int N, int K, void* C,
                        int64_t ldc, int accumulate, hipStream_t stream, float* partial = nullptr,
                        size_t partial_bytes = 0) {
   using Tile = HeadTile<T>;
@@ -440,7 +453,7 @@ static int launch_gemm(const void* A, int64_t lda, int M, const void* B, int64_t
     attr = true;
   }
   GemmParams g;
-  g.A = A; g.B = B; g.C = C; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.A = A; g.B = B; g.C = C; g.a_kslabs = a_kslabs; g.b_kslabs = b_kslabs; g.ldc = ldc;
   g.M = M; g.N = N; g.K = K;
   g.n_mt = (M + 255) / 256; g.n_nt = (N + 255) / 256;
   g.accumulate = accumulate;
@@ -469,8 +482,8 @@ static int launch_gemm(const void* A, int64_t lda, int M, const void* B, int64_t
 template <typename T>
 static int launch_transpose(const T* src, int64_t ld_src, T* dst, int64_t ld_dst, int R, int C, hipStream_t stream) {
   dim3 grid((C + 63) / 64, (int)((ld_dst + 63) / 64));
-  hipLaunchKernelGGL(transpose_pad_kernel<T>, grid, dim3(256), 0, stream, src, ld_src, dst, ld_dst, R, C);
-  return check_launch("transpose_pad_kernel");
+  hipLaunchKernelGGL(transpose_block_kernel<T>, grid, dim3(256), 0, stream, src, ld_src, dst, ld_dst, R, C);
+  return check_launch("transpose_block_kernel");
 }
 
 template <typename T>
@@ -500,7 +513,7 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream, int64_t 
   }
   int rc;
   if (a->dhidden && !(a->weight_t && a->weight_t_ready)) {
-    // WT[h][v] = W[v][h], zero for V <= v < ldv
+    // WT(h, v) = W[v][h], zero for V <= v < ldv, K-blocked
     rc = launch_transpose<T>(weight, H, wt, pl.ldv, (int)V, (int)H, stream);
     if (rc) return rc;
   }
@@ -556,16 +569,16 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream, int64_t 
     }
     if (a->dhidden) {
       // dhidden[chunk][h] = sum_v dz[t][v] WT[h][v]
-      rc = launch_gemm<T, T>(dz, ldz, (int)tc, wt, pl.ldv, (int)H, (int)pl.ldv,
+      rc = launch_gemm<T, T>(dz, ldz / Tile::kSlabK, (int)tc, wt, pl.ldv / Tile::kSlabK, (int)H, (int)pl.ldv,
                              static_cast<T*>(a->dhidden) + c0 * H, H, 0, stream,
                              reinterpret_cast<float*>(ws + pl.off_part), pl.part_bytes);
       if (rc) return rc;
     }
     if (a->dweight) {
-      // hidT[h][t] = hidden[c0 + t][h], zero for tc <= t < ldt;  dW[v][h] (+)= sum_t dzT[v][t] hidT[h][t]
+      // hidT(h, t) = hidden[c0 + t][h], zero for tc <= t < ldt, K-blocked;  dW[v][h] (+)= sum_t dzT(v, t) hidT(h, t)
       rc = launch_transpose<T>(hidden + c0 * H, H, hidt, ldt, (int)tc, (int)H, stream);
       if (rc) return rc;
-      rc = launch_gemm<T, float>(dzt, ldt, (int)V, hidt, ldt, (int)H, (int)ldt, a->dweight, H,
+      rc = launch_gemm<T, float>(dzt, ldt / Tile::kSlabK, (int)V, hidt, ldt / Tile::kSlabK, (int)H, (int)ldt, a->dweight, H,
                                  (a->accumulate_dweight || c0 > 0) ? 1 : 0, stream);
       if (rc) return rc;
     }

@@ -27,7 +27,7 @@ struct FwdParams {
   int T, H, V;
   int n_tb, n_split, tiles_per_split, n_vt;
   float c;  // inv_temperature * log2(e)
-  void* z_out;   // optional [rows][ldz] raw logits in the input dtype
+  void* z_out;   // optional raw logits in the input dtype, K-blocked: rows x ldz, see blocked_index
   int64_t ldz;
   const int32_t* z_row_map;  // optional [T]: destination row per token, < 0: not stored
   int z_rows;                // rows of z_out; mapped rows outside [0, z_rows) are not stored
@@ -118,7 +118,8 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
     const int v1 = v0 + kFwdBM;
     const int next_rows = (p.V - v1) < kFwdBM ? (p.V - v1) : kFwdBM;
     const T* next_w = weight + (int64_t)v1 * p.H;
-    Tile::run(acc, weight + (int64_t)v0 * p.H, p.H, a_rows, hidden, p.H, b_rows, p.H, lds, st,
+    Tile::run(acc, Tile::Operand::row_major(weight + (int64_t)v0 * p.H, p.H, a_rows),
+              Tile::Operand::row_major(hidden, p.H, b_rows), p.H, lds, st,
               (has_next && !kZViaLds) ? next_w : nullptr, next_rows, true);
 
     if (STORE_Z) {
@@ -152,12 +153,13 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
         const int chunk = threadIdx.x & 31;          // 16-byte piece within the 512-byte row
         const int v_idx = v0 + chunk * 8;
         if (v_idx < p.ldz) {
+          const int64_t n_kslab = p.ldz / Tile::kSlabK;
           for (int r = threadIdx.x >> 5; r < kFwdBN; r += Tile::kThreads / 32) {
             const int tok = t0 + r;
             int dst = (tok < p.T) ? (p.z_row_map ? p.z_row_map[tok] : tok) : -1;
             if (dst >= p.z_rows) dst = -1;
             if (dst >= 0)
-              *reinterpret_cast<u32x4*>(z + (int64_t)dst * p.ldz + v_idx) =
+              *reinterpret_cast<u32x4*>(z + blocked_index<T>(dst, v_idx, n_kslab)) =
                   *reinterpret_cast<const u32x4*>(lds + r * kZRow + chunk * 16);
           }
         }
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
               for (int q = 0; q < 4; ++q) {
                 const int v_idx = v0 + wm * WM + mi * 32 + 8 * q + 4 * (lane >> 5);
                 if (v_idx < p.ldz)
-                  *reinterpret_cast<P4*>(z + (int64_t)zrow[ni] * p.ldz + v_idx) =
+                  *reinterpret_cast<P4*>(z + blocked_index<T>(zrow[ni], v_idx, p.ldz / Tile::kSlabK)) =
                       Pack4<T>::make(acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
                                      acc[mi][ni][4 * q + 3]);
               }

@@ -45,15 +45,40 @@ def _stream(t: torch.Tensor):
 
 # --------------------------------------------------------------------------- fused lm_head
 
+def _round_up(x: int, m: int) -> int:
+    return (x + m - 1) // m * m
+
+
 def saved_logits_buffer(T: int, V: int, dtype, device) -> torch.Tensor:
-    """An (uninitialised) [T, ld] buffer the forward can store raw logits in for the backward."""
-    return torch.empty(T, _lib.lib().clgrpo_saved_logits_ld(V), dtype=dtype, device=device)
+    """An (uninitialised) buffer the forward can store raw logits in for the backward: T rows rounded
+    up to whole blocks of 256 by the padded vocabulary extent.  Its layout is the library's K-blocked
+    one (``saved_logits_rowmajor`` turns it back into rows)."""
+    return torch.empty(_round_up(max(T, 1), 256), _lib.lib().clgrpo_saved_logits_ld(V), dtype=dtype, device=device)
+
+
+def _unblock(buf: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
+    """[rows, cols] row-major copy of a K-blocked buffer: blocks of 256 rows, each block holding its
+    128-byte K slabs one after another (slab = 256 rows x 128 bytes)."""
+    e = 128 // buf.element_size()
+    nb, ld = buf.shape[0] // 256, buf.shape[1]
+    return buf.reshape(nb, ld // e, 256, e).permute(0, 2, 1, 3).reshape(nb * 256, ld)[:rows, :cols]
+
+
+def saved_logits_rowmajor(buf: torch.Tensor, rows: int, V: int) -> torch.Tensor:
+    """The first ``rows`` kept rows as an ordinary [rows, V] tensor (a copy; for inspection and tests)."""
+    return _unblock(buf, rows, V)
 
 
 def weight_t_buffer(weight: torch.Tensor) -> torch.Tensor:
-    """An (uninitialised) [H, ld] buffer for W^T that ``lmhead_backward`` can fill once and reuse."""
+    """An (uninitialised) buffer for W^T (K-blocked, H rounded up to 256 rows) that ``lmhead_backward``
+    can fill once and reuse."""
     V, H = weight.shape
-    return torch.empty(H, _lib.lib().clgrpo_saved_logits_ld(V), dtype=weight.dtype, device=weight.device)
+    return torch.empty(_round_up(H, 256), _lib.lib().clgrpo_saved_logits_ld(V), dtype=weight.dtype, device=weight.device)
+
+
+def weight_t_rowmajor(weight_t: torch.Tensor, H: int, V: int) -> torch.Tensor:
+    """W^T as an ordinary [H, V] tensor (a copy; for inspection and tests)."""
+    return _unblock(weight_t, H, V)
 
 
 def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[torch.Tensor],
@@ -96,8 +121,8 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
         saved_logits = _dev(saved_logits, "saved_logits", hidden.dtype)
         if saved_logits.dim() != 2 or not saved_logits.is_contiguous():
             raise ValueError("saved_logits must be a contiguous [rows, ld] tensor")
-        if saved_row_map is None and saved_logits.shape[0] < T:
-            raise ValueError("saved_logits needs at least T rows")
+        if saved_logits.shape[0] % 256 != 0 or (saved_row_map is None and saved_logits.shape[0] < T):
+            raise ValueError("saved_logits must come from saved_logits_buffer with at least T rows")
         ld_saved = saved_logits.shape[1]
         if saved_row_map is not None:
             saved_row_map = _dev(saved_row_map, "saved_row_map", torch.int32)
@@ -202,12 +227,13 @@ def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=N
     ld_saved, has_saved = 0, 0
     if saved_logits is not None:
         saved_logits = _dev(saved_logits, "saved_logits", hidden.dtype)
-        if saved_logits.dim() != 2 or saved_logits.shape[0] < T or not saved_logits.is_contiguous():
-            raise ValueError("saved_logits must be a contiguous [>=T, ld] tensor")
+        if saved_logits.dim() != 2 or saved_logits.shape[0] < T or saved_logits.shape[0] % 256 != 0 \
+                or not saved_logits.is_contiguous():
+            raise ValueError("saved_logits must come from saved_logits_buffer with at least T rows")
         ld_saved, has_saved = saved_logits.shape[1], 1
     if weight_t is not None:
         weight_t = _dev(weight_t, "weight_t", hidden.dtype)
-        if tuple(weight_t.shape) != (H, L.clgrpo_saved_logits_ld(V)) or not weight_t.is_contiguous():
+        if tuple(weight_t.shape) != (_round_up(H, 256), L.clgrpo_saved_logits_ld(V)) or not weight_t.is_contiguous():
             raise ValueError("weight_t must come from weight_t_buffer(weight)")
     if chunk_tokens is None:
         chunk_tokens = T

@@ -58,15 +58,20 @@ typedef struct {
   float* lse;              /* [T] out, fp32 (logsumexp_v z); required */
   void* workspace;
   size_t workspace_bytes;
-  void* saved_logits;      /* optional out [T][ld_saved] in `dtype`: the raw logits hidden.W^T (before the
-                              temperature), for a later clgrpo_lmhead_bwd of the SAME T rows that then skips
-                              the recomputation.  NULL: nothing is stored.  Callers bound its size by
-                              processing a micro-batch in token chunks. */
-  int64_t ld_saved;        /* row stride in elements, a multiple of 64, >= clgrpo_saved_logits_ld(V) */
+  void* saved_logits;      /* optional out, `dtype`: the raw logits hidden.W^T (before the temperature), for a
+                              later clgrpo_lmhead_bwd of the SAME rows that then skips the recomputation.
+                              NULL: nothing is stored.  Callers bound its size by processing a micro-batch in
+                              token chunks.  The buffer is opaque to the caller: ceil(rows / 256) * 256 rows of
+                              ld_saved elements, laid out in blocks of 256 rows; inside a block the 128-byte K
+                              slabs of all 256 rows follow one another, so element (row, k) lives at
+                              (((row / 256) * (ld_saved / E) + k / E) * 256 + row % 256) * E + k % E,
+                              E = 128 / sizeof(dtype).  This is the operand layout of the backward GEMMs. */
+  int64_t ld_saved;        /* K extent in elements, a multiple of 64, >= clgrpo_saved_logits_ld(V) */
   const int32_t* saved_row_map; /* optional [T]: row of saved_logits that receives token t's logits, or a
                               negative value to store nothing for t (tokens whose upstream gradient is
                               known to be zero, e.g. masked-out prompt positions).  NULL: row t. */
-  int64_t saved_rows;      /* rows of saved_logits; a mapped row outside [0, saved_rows) is not stored */
+  int64_t saved_rows;      /* rows the buffer can address (a multiple of 256 is allocated; see above); a
+                              mapped row outside [0, saved_rows) is not stored */
 } clgrpo_lmhead_fwd_args;
 
 /* Row stride (elements) the saved-logits buffer must have: V rounded up to 64. */
@@ -99,11 +104,13 @@ typedef struct {
   int32_t accumulate_dweight; /* nonzero: dweight += ; zero: dweight = */
   void* workspace;
   size_t workspace_bytes;   /* sets the token chunk: see clgrpo_lmhead_bwd_workspace_bytes */
-  void* saved_logits;       /* optional in/out [T][ld_saved]: logits stored by clgrpo_lmhead_fwd for these
-                               rows.  Overwritten in place with d(logits); the recomputation is skipped. */
+  void* saved_logits;       /* optional in/out: logits stored by clgrpo_lmhead_fwd for these rows (same opaque
+                               blocked layout, ceil(T / 256) * 256 rows of ld_saved elements).  Overwritten in
+                               place with d(logits); the recomputation is skipped. */
   int64_t ld_saved;
-  void* weight_t;           /* optional [H][clgrpo_saved_logits_ld(V)] in `dtype`: caller-kept W^T, so that
-                               several calls with the same weight (token chunks of one step) build it once */
+  void* weight_t;           /* optional, `dtype`: caller-kept W^T in the same blocked layout (ceil(H / 256) * 256
+                               rows of clgrpo_saved_logits_ld(V) elements), so that several calls with the same
+                               weight (token chunks of one step) build it once */
   int32_t weight_t_ready;   /* zero: this call fills weight_t; nonzero: it already holds W^T */
 } clgrpo_lmhead_bwd_args;
 

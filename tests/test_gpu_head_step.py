@@ -103,8 +103,8 @@ def test_kept_logits_backward_equals_recompute(dev):
     lp2, ent2, _, lse2 = ops.lmhead_forward(hidden, weight, labels, 0.8)
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2)            # storing logits does not change the statistics
     z = torch.nn.functional.linear(hidden.float(), weight.float())
-    assert_close_rel(zbuf[:, :V], z, 2 ** -8, "stored logits")        # bf16 rounding of the raw logits
-    assert (zbuf[:, V:] == 0).all()
+    assert_close_rel(ops.saved_logits_rowmajor(zbuf, T, V), z, 2 ** -8, "stored logits")   # bf16 rounding of the raw logits
+    assert (ops.saved_logits_rowmajor(zbuf, T, zbuf.shape[1])[:, V:] == 0).all()         # vocabulary padding columns
     dh1, dw1 = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_en, 0.8)
     dh2, dw2 = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_en, 0.8, saved_logits=zbuf)
     assert_close_rel(dh2, dh1, 1e-2, "dhidden kept vs recompute")
@@ -124,7 +124,8 @@ def test_weight_transpose_cache_is_reused_across_micro_batches(dev):
     cache = {}
     first = grpo_head_step(*args, weight_t_cache=cache, **kw)
     wt = cache["weight_t"]
-    assert torch.equal(wt[:, :weight.shape[0]], args[1].t())
+    from chatlearn_amd import ops
+    assert torch.equal(ops.weight_t_rowmajor(wt, weight.shape[1], weight.shape[0]), args[1].t())
     second = grpo_head_step(*args, weight_t_cache=cache, **kw)
     assert cache["weight_t"] is wt
     for out in (first, second):
