@@ -363,22 +363,32 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, int k_sp
 }
 
 // dst(c, r) = src[r][c] for r < R, c < C and 0 for R <= r < ld_dst, where dst is the K-blocked
-// operand with C rows and ld_dst K elements (see blocked_index).  64x64 tiles.
+// operand with C rows and ld_dst K elements (see blocked_index).  64x64 tiles, 16-byte accesses on
+// both sides (C and ld_src are multiples of 32 elements here, so a 16-byte piece never straddles an edge).
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_block_kernel(const T* __restrict__ src, int64_t ld_src,
                                                               T* __restrict__ dst, int64_t ld_dst, int R, int C) {
-  __shared__ T tile[64][65];
+  constexpr int VEC = 16 / (int)sizeof(T);       // elements per 16-byte access
+  constexpr int CPR = 64 / VEC;                  // accesses per 64-wide tile row
+  constexpr int RPP = 256 / CPR;                 // tile rows covered per pass
   constexpr int kE = kRowBytes / (int)sizeof(T);
+  __shared__ T tile[64][64 + VEC];               // [c][r], padded rows
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  for (int i = ty; i < 64; i += 4) {
-    const int r = r0 + i, c = c0 + tx;
-    tile[i][tx] = (r < R && c < C) ? src[(int64_t)r * ld_src + c] : (T)0.f;
+  const int q = threadIdx.x % CPR, row = threadIdx.x / CPR;
+  for (int rr = row; rr < 64; rr += RPP) {
+    const int r = r0 + rr, c = c0 + q * VEC;
+    alignas(16) T vals[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) vals[j] = (T)0.f;
+    if (r < R && c < C) *reinterpret_cast<u32x4*>(vals) = *reinterpret_cast<const u32x4*>(src + (int64_t)r * ld_src + c);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) tile[q * VEC + j][rr] = vals[j];
   }
   __syncthreads();
-  for (int i = ty; i < 64; i += 4) {
-    const int c = c0 + i, r = r0 + tx;
-    if (c < C && r < ld_dst) dst[blocked_index<T>(c, r, ld_dst / kE)] = tile[tx][i];
+  for (int cc = row; cc < 64; cc += RPP) {
+    const int c = c0 + cc, r = r0 + q * VEC;
+    if (c < C && r < ld_dst)
+      *reinterpret_cast<u32x4*>(dst + blocked_index<T>(c, r, ld_dst / kE)) = *reinterpret_cast<const u32x4*>(&tile[cc][q * VEC]);
   }
 }
 
