@@ -402,7 +402,8 @@ int validate_head_shape(const char* who, int64_t T, int64_t H, int64_t V, int32_
                                              (long long)T, (long long)H, (long long)V);
   const int slab = dtype == CLGRPO_BF16 ? 64 : 32;
   if (H % slab != 0) return fail(CLGRPO_ESHAPE, "%s: H=%lld must be a multiple of %d", who, (long long)H, slab);
-  if (T >= (1LL << 30) || V >= (1LL << 30) || H >= (1LL << 24)) return fail(CLGRPO_ESHAPE, "%s: size too large", who);
+  // 256 rows of H elements must stay below 2^31 bytes (32-bit offsets of the buffer loads)
+  if (T >= (1LL << 30) || V >= (1LL << 30) || H > (1LL << 20)) return fail(CLGRPO_ESHAPE, "%s: size too large", who);
   return CLGRPO_OK;
 }
 
