@@ -205,6 +205,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
             if not acc_dw:
                 dw = torch.zeros(V, hidden.shape[1], dtype=torch.float32, device=hidden.device) if dw is None \
                     else dw.zero_()
+            rows_projected_bwd -= n
         else:
             pick = lambda x: None if x is None else ops.gather_rows(x.reshape(n, -1), live).reshape(-1)
             if h_c is None:

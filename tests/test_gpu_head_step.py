@@ -134,3 +134,36 @@ def test_weight_transpose_cache_is_reused_across_micro_batches(dev):
     cache["weight_t"] = torch.zeros_like(wt)
     stale = grpo_head_step(*args, weight_t_cache=cache, **kw)
     assert (stale["dhidden"] == 0).all()
+
+
+def test_empty_and_fully_masked_inputs(dev):
+    """Edge cases the trainer can produce: no tokens at all, and a micro-batch whose loss mask is
+    all zero (every response truncated away): zero loss sums, zero gradients, nothing projected."""
+    from chatlearn_amd import ops
+    from chatlearn_amd.fused import grpo_head_step
+    H, V = 128, 1000
+    g = torch.Generator().manual_seed(4)
+    weight = (torch.randn(V, H, generator=g) * 0.05).bfloat16().to(dev)
+    empty = torch.empty(0, H, dtype=torch.bfloat16, device=dev)
+    lp, ent, mx, lse = ops.lmhead_forward(empty, weight, torch.empty(0, dtype=torch.int64, device=dev))
+    assert lp.numel() == ent.numel() == lse.numel() == 0
+    dh, dw = ops.lmhead_backward(empty, weight, torch.empty(0, dtype=torch.int64, device=dev), lse, None, lp)
+    assert dh.shape == (0, H) and (dw == 0).all()
+
+    T = 300
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    labels = torch.randint(0, V, (T,), generator=g).to(dev)
+    zeros = torch.zeros(T, device=dev)
+    cu = torch.tensor([0, 100, 300], dtype=torch.int32, device=dev)
+    out = grpo_head_step(hidden, weight, labels, zeros, zeros, torch.tensor([1.0, -1.0], device=dev), cu,
+                         torch.zeros(T, dtype=torch.int32, device=dev), n_tokens_total=1.0, kl_coef=1e-3,
+                         cu_seqlens_host=[0, 100, 300])
+    assert out["rows_projected_bwd"] == 0 and float(out["num_masked"]) == 0
+    assert float(out["sums"][0]) == 0 and float(out["sums"][1]) == 0
+    assert (out["dhidden"] == 0).all() and (out["dweight"] == 0).all()
+    assert torch.isfinite(out["logprob"]).all()
+    # a label outside the vocabulary has no logit: NaN logprob, not a silent number
+    bad = labels.clone()
+    bad[5] = V + 3
+    lp_bad, *_ = ops.lmhead_forward(hidden, weight, bad)
+    assert torch.isnan(lp_bad[5]) and torch.isfinite(lp_bad[:5]).all()
