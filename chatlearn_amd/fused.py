@@ -74,22 +74,33 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
 
 
 def _token_chunks(T, chunk_tokens, seq_bounds):
-    """[lo, hi) token ranges of about ``chunk_tokens`` tokens.  With ``seq_bounds`` (the host copy of
-    cu_seqlens) every range ends on a sequence boundary, growing past the target where one
-    sequence is longer than it."""
+    """[lo, hi) token ranges of at most ``chunk_tokens`` tokens, as few as that allows and of about
+    equal size (a small last range would run the backward GEMMs at poor efficiency).  With
+    ``seq_bounds`` (the host copy of cu_seqlens) every range ends on a sequence boundary; a range
+    exceeds ``chunk_tokens`` only where a single sequence is longer than it."""
     if chunk_tokens is None or chunk_tokens >= T:
         return [(0, T)]
-    if seq_bounds is None:
-        return [(lo, min(T, lo + chunk_tokens)) for lo in range(0, T, chunk_tokens)]
+    cuts = sorted(set(int(x) for x in seq_bounds if 0 < int(x) < T)) + [T] if seq_bounds is not None else None
+    # number of ranges a greedy fill needs: the balanced cut below aims at that many
+    n, lo = 0, 0
+    while lo < T:
+        if cuts is None:
+            lo = min(T, lo + chunk_tokens)
+        else:
+            ok = [c for c in cuts if lo < c <= lo + chunk_tokens]
+            lo = max(ok) if ok else min(c for c in cuts if c > lo)
+        n += 1
     out, lo = [], 0
-    for b in range(1, len(seq_bounds)):
-        nxt = seq_bounds[b + 1] if b + 1 < len(seq_bounds) else None
-        if nxt is None or nxt - lo > chunk_tokens:
-            if seq_bounds[b] > lo:
-                out.append((lo, seq_bounds[b]))
-                lo = seq_bounds[b]
-    if lo < T:
-        out.append((lo, T))
+    while lo < T:
+        left = max(-(-(T - lo) // chunk_tokens), n - len(out), 1)
+        target = lo + -(-(T - lo) // left)
+        if cuts is None:
+            hi = min(T, target)
+        else:
+            ok = [c for c in cuts if lo < c <= lo + chunk_tokens]
+            hi = min(ok, key=lambda c: (abs(c - target), c)) if ok else min(c for c in cuts if c > lo)
+        out.append((lo, hi))
+        lo = hi
     return out
 
 
