@@ -87,7 +87,8 @@ class ThdPackArgs(C.Structure):
     _fields_ = [("B", i64), ("S", i64), ("tokens", vp), ("prompt_len", vp), ("response_len", vp),
                 ("align", i32), ("cp_size", i32), ("cp_rank", i32), ("pad_token", i64), ("total_padded", i64),
                 ("cu_seqlens_padded", vp), ("seqlens", vp), ("seqlens_padded", vp), ("stats", vp), ("status", vp),
-                ("indices", vp), ("seq_indices", vp), ("out_tokens", vp), ("out_labels", vp), ("out_loss_mask", vp)]
+                ("indices", vp), ("seq_indices", vp), ("out_tokens", vp), ("out_labels", vp), ("out_loss_mask", vp),
+                ("out_position_ids", vp)]
 
 
 class RowsArgs(C.Structure):

@@ -68,16 +68,31 @@ class PolicyStep:
             if 'loss_mask' in data_b:
                 loss_mask = data_b['loss_mask']
             indices = cu_seqlens = None
-            if self.packing:
-                tokens_, indices, cu_seqlens, _ = unpad_input(tokens_.unsqueeze(-1).to(self.device),
-                                                              attn_mask.to(self.device))
-                tokens_ = tokens_.permute(1, 0)
-                position_ids, *_ = unpad_input(position_ids.unsqueeze(-1).to(self.device), attn_mask.to(self.device))
-                position_ids = position_ids.permute(1, 0)
-            tokens = tokens_
-            # labels roll along the (packed or padded) token row; the training mask rolls along the
-            # padded rows and loses its last column (policy_trainer.py:135,160-162)
-            labels, _ = ops.shift_labels(tokens.to(self.device).contiguous(), None, zero_last=False)
+            if self.packing and 'position_ids' not in data_b:
+                # unpad_input of tokens and position ids plus the label roll (policy_trainer.py:143-162) in
+                # one device pass driven by the length lists; no device value is read back
+                packed = ops.thd_pack(tokens_.to(self.device), data_b["prompt_token_length"],
+                                      data_b["response_token_length"], align=1, pad_token=0,
+                                      want_loss_mask=False, want_position_ids=True, verify_on_device=False)
+                tokens = packed["tokens"].unsqueeze(0)
+                position_ids = packed["position_ids"].unsqueeze(0)
+                labels = packed["labels"].unsqueeze(0)
+                indices, cu_seqlens = packed["indices"], packed["cu_seqlens_padded"]
+                width = packed["max_seqlen_padded"]
+                if width != ori_seq_len:      # the batch is padded wider than its longest sample
+                    indices = (indices // width) * ori_seq_len + indices % width
+            else:
+                if self.packing:
+                    tokens_, indices, cu_seqlens, _ = unpad_input(tokens_.unsqueeze(-1).to(self.device),
+                                                                  attn_mask.to(self.device))
+                    tokens_ = tokens_.permute(1, 0)
+                    position_ids, *_ = unpad_input(position_ids.unsqueeze(-1).to(self.device),
+                                                   attn_mask.to(self.device))
+                    position_ids = position_ids.permute(1, 0)
+                tokens = tokens_
+                # labels roll along the (packed or padded) token row (policy_trainer.py:135,160)
+                labels, _ = ops.shift_labels(tokens.to(self.device).contiguous(), None, zero_last=False)
+            # the training mask rolls along the padded rows and loses its last column (policy_trainer.py:161-162)
             shifted = None
             if training:
                 _, shifted = ops.shift_labels(None, loss_mask.to(self.device).to(torch.int32).contiguous(),

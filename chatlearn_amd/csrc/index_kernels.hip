@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void thd_offsets_kernel(int64_t B, int64_t S, 
     seqlens[b] = (int32_t)len;
     padded[b] = (int32_t)pad;
     if (len > S || len < 0) flag |= 2;
-    if (pad % (2 * cp_size) != 0) flag |= 4;
+    if (cp_size > 1 && pad % (2 * cp_size) != 0) flag |= 4;   // one rank keeps everything: any length will do
     sum += pad;
     mx = pad > mx ? (int32_t)pad : mx;
   }
@@ -234,6 +234,7 @@ struct ThdFill {
   int64_t* out_tokens;
   int64_t* out_labels;
   int32_t* out_loss_mask;
+  int64_t* out_position_ids;
 };
 
 __device__ __forceinline__ void thd_at(const ThdFill& p, int64_t pos, int64_t& token, int& in_loss, int& seq, int64_t& j) {
@@ -267,6 +268,7 @@ __global__ __launch_bounds__(256) void thd_fill_kernel(ThdFill p) {
       int il, ns;
       thd_at(p, src, tk, il, ns, nj);
       p.out_tokens[i] = tk;
+      if (p.out_position_ids) p.out_position_ids[i] = nj;
       thd_at(p, src + 1 == p.total ? 0 : src + 1, tk, il, ns, nj);
       p.out_labels[i] = tk;
       if (p.out_loss_mask) p.out_loss_mask[i] = il;
@@ -406,6 +408,7 @@ extern "C" int clgrpo_thd_pack(const clgrpo_thd_pack_args* a, void* stream) {
   f.out_tokens = a->out_tokens;
   f.out_labels = a->out_labels;
   f.out_loss_mask = a->out_loss_mask;
+  f.out_position_ids = a->out_position_ids;
   hipLaunchKernelGGL(thd_fill_kernel, dim3(grid_for(a->total_padded, 256)), dim3(256), 0, s, f);
   return check_launch("thd_fill_kernel");
 }

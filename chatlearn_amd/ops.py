@@ -450,7 +450,8 @@ def unpad_indices(attn_mask: torch.Tensor):
 
 
 def thd_pack(tokens: torch.Tensor, prompt_len, response_len, align: int, pad_token: int, cp_size: int = 1,
-             cp_rank: int = 0, want_loss_mask: bool = True) -> Dict[str, object]:
+             cp_rank: int = 0, want_loss_mask: bool = True, want_position_ids: bool = False,
+             verify_on_device: bool = True) -> Dict[str, object]:
     """Packed (THD) micro-batch from per-sample lengths, in one device pass.
 
     ``tokens`` int64 [B, S] on the device; ``prompt_len`` / ``response_len`` host sequences (or CPU
@@ -458,9 +459,10 @@ def thd_pack(tokens: torch.Tensor, prompt_len, response_len, align: int, pad_tok
     read back to size the outputs.  Every sequence is padded with ``pad_token`` to a multiple of
     ``align``.  Returns a dict: ``cu_seqlens_padded`` int32 [B+1], ``seqlens`` / ``seqlens_padded`` int32
     [B], ``indices`` int64 [total] (positions in the padded [B, max padded length] layout),
-    ``seq_indices`` / ``tokens`` / ``labels`` int64 [total / cp_size] and ``loss_mask`` int32 for this
-    context-parallel rank, ``num_loss_tokens`` (device int32 scalar), ``total_padded`` and
-    ``max_seqlen_padded`` (host ints).  Raises if the device-side sizes disagree with the host's."""
+    ``seq_indices`` / ``tokens`` / ``labels`` (/ ``position_ids``) int64 [total / cp_size] and ``loss_mask`` int32
+    for this context-parallel rank, ``num_loss_tokens`` (device int32 scalar), ``total_padded`` and
+    ``max_seqlen_padded`` (host ints).  The lengths are checked on the host; with ``verify_on_device`` the
+    device's own consistency word is read back as well (one host round trip)."""
     tokens = _dev(tokens, "tokens", torch.int64)
     if tokens.dim() != 2:
         raise ValueError("tokens must be [B, S]")
@@ -472,7 +474,11 @@ def thd_pack(tokens: torch.Tensor, prompt_len, response_len, align: int, pad_tok
     align, cp_size, cp_rank = int(align), int(cp_size), int(cp_rank)
     if align <= 0 or cp_size <= 0:
         raise ValueError("align and cp_size must be positive")
+    if any(p < 0 or r < 0 or p + r > S for p, r in zip(pl, rl)):
+        raise ValueError("thd_pack: a sequence is longer than S (or a length is negative)")
     padded = [(p + r + align - 1) // align * align for p, r in zip(pl, rl)]
+    if any(x % (2 * cp_size) for x in padded) and cp_size > 1:
+        raise ValueError("thd_pack: a padded length is not a multiple of 2*cp_size")
     total, max_padded = sum(padded), max(padded)
     dev = tokens.device
     i32 = dict(dtype=torch.int32, device=dev)
@@ -484,17 +490,20 @@ def thd_pack(tokens: torch.Tensor, prompt_len, response_len, align: int, pad_tok
     indices, seq_indices = torch.empty(total, **i64o), torch.empty(per_rank, **i64o)
     out_tokens, out_labels = torch.empty(per_rank, **i64o), torch.empty(per_rank, **i64o)
     out_mask = torch.empty(per_rank, **i32) if want_loss_mask else None
+    out_pos = torch.empty(per_rank, **i64o) if want_position_ids else None
     a = _lib.ThdPackArgs(B, S, _ptr(tokens), _ptr(lens[0]), _ptr(lens[1]), align, cp_size, cp_rank, int(pad_token), total,
                          _ptr(cu), _ptr(seqlens), _ptr(seqlens_padded), _ptr(stats), _ptr(status), _ptr(indices),
-                         _ptr(seq_indices), _ptr(out_tokens), _ptr(out_labels), _ptr(out_mask))
+                         _ptr(seq_indices), _ptr(out_tokens), _ptr(out_labels), _ptr(out_mask), _ptr(out_pos))
     _lib.call("clgrpo_thd_pack", a, _stream(tokens))
-    bad = int(status.item())
+    # the device recomputes the sizes from the same lengths; reading its verdict costs a host round trip
+    bad = int(status.item()) if verify_on_device else 0
     if bad:
         why = [m for bit, m in ((1, "padded total differs from the host's"), (2, "a sequence is longer than S"),
                                 (4, "a padded length is not a multiple of 2*cp_size")) if bad & bit]
         raise ValueError("thd_pack: " + "; ".join(why))
     return {"cu_seqlens_padded": cu, "seqlens": seqlens, "seqlens_padded": seqlens_padded, "indices": indices,
             "seq_indices": seq_indices, "tokens": out_tokens, "labels": out_labels, "loss_mask": out_mask,
+            "position_ids": out_pos,
             "num_loss_tokens": stats[2], "total_padded": total, "max_seqlen_padded": max_padded}
 
 

@@ -291,8 +291,8 @@ int clgrpo_unpad_indices(const clgrpo_unpad_indices_args* a, void* stream);
  * Row i of the padded batch holds seqlen_i = prompt_i + response_i tokens; its packed segment has
  * padded_i = ceil(seqlen_i / align) * align tokens.  The caller passes total_padded = sum padded_i
  * (known on the host from the same lengths); the call fails the `status` word (bit 0) if the device
- * sum disagrees, (bit 1) if a sequence is longer than S, (bit 2) if a padded length is not a
- * multiple of 2*cp_size.
+ * sum disagrees, (bit 1) if a sequence is longer than S, (bit 2) if cp_size > 1 and a padded length is
+ * not a multiple of 2*cp_size.
  * Outputs over the whole packed row (n = total_padded):
  *   cu_seqlens_padded [B+1], seqlens [B], seqlens_padded [B]            int32
  *   stats[0] = total_padded, stats[1] = max padded length                int32
@@ -303,6 +303,8 @@ int clgrpo_unpad_indices(const clgrpo_unpad_indices_args* a, void* stream);
  *   tokens [m], labels [m] (packed row rolled left by one, wrapping)    int64
  *   loss_mask [m] (rolled the same way)                                  int32
  *   stats[2] = number of ones in loss_mask                               int32
+ * With align = 1 and cp_size = 1 this is also the packing step of the FSDP trainer (unpad_input of the
+ * tokens and position ids plus the label roll, policy_trainer.py:143-162) without its host round trip.
  */
 typedef struct {
   int64_t B, S;
@@ -323,6 +325,8 @@ typedef struct {
   int64_t* out_tokens;          /* [total_padded / cp_size] out */
   int64_t* out_labels;          /* [total_padded / cp_size] out */
   int32_t* out_loss_mask;       /* [total_padded / cp_size] out, or NULL */
+  int64_t* out_position_ids;    /* [total_padded / cp_size] out, or NULL: position of the token inside its sequence
+                                   (what unpad_input gives for the padded arange position ids, policy_trainer.py:152-156) */
 } clgrpo_thd_pack_args;
 int clgrpo_thd_pack(const clgrpo_thd_pack_args* a, void* stream);
 

@@ -112,3 +112,23 @@ def test_thd_pack_against_hand_worked_cases(dev):
         assert got["labels"].tolist() == c["labels"]
         assert got["loss_mask"].tolist() == c["loss_mask"]
         assert int(got["num_loss_tokens"]) == c["num_tokens"]
+
+
+def test_thd_pack_with_align_one_is_the_fsdp_packing_step(dev):
+    """align = 1: tokens and position ids as unpad_input leaves them, labels rolled along the packed
+    row, indices into the padded [B, S] batch (policy_trainer.py:143-162)."""
+    from chatlearn_amd import ops
+    tokens, p, r = _batch(7, 90, seed=21)
+    S = max(a + b for a, b in zip(p, r))
+    tokens = tokens[:, :S].contiguous()
+    attn, _, pos = oidx.generate_loss_mask_position_ids(tokens, p, r)
+    want_tok, want_idx, want_cu, _ = oidx.unpad_input(tokens.unsqueeze(-1), attn)
+    want_pos = oidx.unpad_input(pos.unsqueeze(-1), attn)[0]
+    got = ops.thd_pack(tokens.to(dev), p, r, align=1, pad_token=0, want_loss_mask=False, want_position_ids=True,
+                       verify_on_device=False)
+    assert got["max_seqlen_padded"] == S
+    assert torch.equal(got["tokens"].cpu(), want_tok[:, 0])
+    assert torch.equal(got["position_ids"].cpu(), want_pos[:, 0])
+    assert torch.equal(got["indices"].cpu(), want_idx)
+    assert torch.equal(got["cu_seqlens_padded"].cpu(), want_cu)
+    assert torch.equal(got["labels"].cpu(), torch.roll(want_tok[:, 0], shifts=-1))
