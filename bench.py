@@ -308,6 +308,23 @@ def main():
         "step_mfma_frac": step_flops / dt / 1e12 / peak,
         "stage_ms": {"forward": fwd_ms, "loss": loss_ms, "backward": bwd_ms},
     }
+    if train and mask is not None and not args.skip_masked_forward and not args.no_skip_masked:
+        # Reported beside the headline, never as `value`: the same step with the rows outside the loss
+        # mask also left out of the forward (their per-token outputs become zero, loss and gradients
+        # are unchanged).
+        args.skip_masked_forward = True
+        for _ in range(max(1, args.warmup // 2)):
+            lean = step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            lean = step()
+        torch.cuda.synchronize()
+        l_dt = (time.perf_counter() - t1) / args.steps
+        args.skip_masked_forward = False
+        out["variant_skip_masked_forward"] = {"tokens_per_s": T / l_dt, "ms_per_step": l_dt * 1e3,
+                                              "T_projected_forward": lean["rows_projected_fwd"],
+                                              "T_projected_backward": lean["rows_projected_bwd"]}
     if not args.no_unfused and train:
         try:
             u_dt = unfused_gpu(cfg, hidden, weight, labels, old, ref, adv, cu, mask, n_tok, max(2, args.steps // 3))
