@@ -11,7 +11,15 @@
 // undone by the fragment reads.  Two LDS stages: while the matrix cores work on
 // stage s, the next slab lands in stage s^1; one workgroup barrier per slab,
 // placed before the last K-step so that step's matrix instructions cover the
-// first fragment reads of the next slab.
+// first fragment reads of the next slab; that barrier is preceded by an
+// explicit wait for the wave's outstanding loads, because a barrier alone does
+// not wait for loads whose destination is LDS.
+//
+// Operands are either row-major (the caller's hidden states and weight) or
+// K-blocked (the library's own intermediates: per tile and slab one contiguous
+// 32 KB piece, see Operand).  Consecutive K loops of a workgroup that keep the
+// same B rows can stream into each other: the last two slab periods of one loop
+// already request the first two slabs of the next (see Stream).
 //
 // Accumulator layout (v_mfma_f32_32x32x*): for the 32x32 block (mi, ni) of a
 // wave, lane l, register r hold
