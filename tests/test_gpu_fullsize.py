@@ -139,3 +139,32 @@ def test_other_benchmark_configs_at_full_size(dev, name):
     assert (lp <= 0).all() and (ent > 0).all() and (ent <= math.log(cfg.V) + 1e-3).all()
     assert_close_rel(lp[rows], want[0], 1e-2, "logprob sample")
     assert_close_rel(ent[rows], want[1], 1e-2, "entropy sample")
+
+
+def test_vocabulary_shards_merge_to_the_unsharded_result_at_full_size(dev, big):
+    """Four tensor-parallel ranks' shares of the Qwen3-8B head, run one after another on this GPU:
+    the merged records reproduce the unsharded statistics and the shard gradients add up."""
+    from chatlearn_amd import ops
+    T = 4096                                              # a quarter of the micro-batch keeps this quick
+    hidden, labels, weight = big["hidden"][:T], big["labels"][:T], big["weight"]
+    V, n = CFG.V, 4
+    per = V // n
+    lp0, ent0, mx0, lse0 = ops.lmhead_forward(hidden, weight, labels)
+    records = torch.stack([ops.lmhead_forward_shard(hidden, weight[r * per:(r + 1) * per], labels, r * per) for r in range(n)])
+    lp, ent, mx, lse = ops.lmhead_merge_shards(records, labels, V)
+    assert torch.equal(mx, mx0)
+    assert (lp - lp0).abs().max() < 1e-4 and (ent - ent0).abs().max() < 1e-4 and (lse - lse0).abs().max() < 1e-4
+    g = torch.Generator(device=dev).manual_seed(2)
+    g_lp = torch.randn(T, generator=g, device=dev) * big["mask"][:T]
+    dh0, dw0 = ops.lmhead_backward(hidden, weight, labels, lse0, None, g_lp)
+    dh = torch.zeros(T, CFG.H, dtype=torch.float32, device=dev)
+    for r in (0, n - 1):                                  # first and last shard: dW rows equal the unsharded ones
+        dh_r, dw_r = ops.lmhead_backward(hidden, weight[r * per:(r + 1) * per], labels, lse, None, g_lp,
+                                         vocab_begin=r * per)
+        assert_close_rel(dw_r, dw0[r * per:(r + 1) * per], 1e-2, f"dW rows of shard {r}")
+        dh += dh_r.float()
+    for r in range(1, n - 1):
+        dh_r, _ = ops.lmhead_backward(hidden, weight[r * per:(r + 1) * per], labels, lse, None, g_lp,
+                                      need_dweight=False, vocab_begin=r * per)
+        dh += dh_r.float()
+    assert_close_rel(dh, dh0.float(), 1e-2, "sum of the shards' dhidden")
