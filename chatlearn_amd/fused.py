@@ -22,13 +22,27 @@ from ._lib import LOSS_GRPO, LOSS_GSPO
 
 class _FusedHead(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, labels, temperature, need_entropy, dweight_buffer):
-        lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, temperature, need_entropy)
+    def forward(ctx, hidden, weight, labels, temperature, need_entropy, dweight_buffer, keep_logits, row_mask):
+        T = hidden.shape[0]
+        zbuf = live = row_map = None
+        if keep_logits and T > 0:
+            if row_mask is not None:
+                # rows outside the mask get a zero upstream gradient whatever their logits are:
+                # keep logits only for the others and run the backward on that compact set
+                live, _, _, _ = ops.unpad_indices(row_mask.reshape(1, T))
+                row_map = torch.full((T,), -1, dtype=torch.int32, device=hidden.device)
+                row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
+            rows = T if live is None else int(live.numel())
+            if rows > 0:
+                zbuf = ops.saved_logits_buffer(rows, weight.shape[0], hidden.dtype, hidden.device)
+        lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, temperature, need_entropy,
+                                             saved_logits=zbuf, saved_row_map=row_map if zbuf is not None else None)
         ctx.save_for_backward(hidden, weight, labels, lse, ent if ent is not None else lse)
         ctx.set_materialize_grads(False)
         ctx.temperature = temperature
         ctx.has_entropy = ent is not None
         ctx.dweight_buffer = dweight_buffer
+        ctx.zbuf, ctx.live = zbuf, live
         if ent is None:
             ent = torch.zeros(0, device=hidden.device)
             ctx.mark_non_differentiable(ent)
@@ -38,25 +52,43 @@ class _FusedHead(torch.autograd.Function):
     def backward(ctx, g_lp, g_ent):
         hidden, weight, labels, lse, ent = ctx.saved_tensors
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        zbuf, live = ctx.zbuf, ctx.live
+        ctx.zbuf = None                      # the buffer is consumed (overwritten) by this backward
+        none = (None,) * 8
         if g_lp is None and g_ent is None:
-            return None, None, None, None, None, None
+            return none
         if g_lp is None:
             g_lp = torch.zeros_like(lse)
         use_ent = ctx.has_entropy and g_ent is not None
-        dh, dw = ops.lmhead_backward(
-            hidden, weight, labels, lse, ent if use_ent else None, g_lp.float().contiguous(),
-            g_ent.float().contiguous() if use_ent else None, ctx.temperature,
-            need_dhidden=need_h, need_dweight=need_w, dweight=ctx.dweight_buffer,
-            accumulate_dweight=ctx.dweight_buffer is not None)
+        g_lp = g_lp.float().contiguous()
+        g_ent = g_ent.float().contiguous() if use_ent else None
+        ent = ent if use_ent else None
+        T = hidden.shape[0]
+        kw = dict(need_dhidden=need_h, need_dweight=need_w, dweight=ctx.dweight_buffer,
+                  accumulate_dweight=ctx.dweight_buffer is not None)
+        if live is None:
+            dh, dw = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_ent, ctx.temperature,
+                                         saved_logits=zbuf, **kw)
+        elif live.numel() == 0:
+            dh = torch.zeros_like(hidden) if need_h else None
+            dw = None
+            if need_w and ctx.dweight_buffer is None:
+                dw = torch.zeros(weight.shape, dtype=torch.float32, device=hidden.device)
+        else:
+            pick = lambda x: None if x is None else ops.gather_rows(x.reshape(T, -1), live).reshape(-1)
+            dh_c, dw = ops.lmhead_backward(ops.gather_rows(hidden, live), weight, pick(labels), pick(lse), pick(ent),
+                                           pick(g_lp), pick(g_ent), ctx.temperature, saved_logits=zbuf, **kw)
+            dh = ops.scatter_rows(dh_c, live, T) if need_h else None
         if dw is not None:
             # A caller-supplied fp32 main-grad buffer was accumulated in place; autograd gets no copy.
             dw = None if ctx.dweight_buffer is not None else dw.to(weight.dtype)
-        return dh, dw, None, None, None, None
+        return (dh, dw) + (None,) * 6
 
 
 def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, *,
                                  temperature: float = 1.0, need_entropy: bool = True,
-                                 dweight_buffer: Optional[torch.Tensor] = None):
+                                 dweight_buffer: Optional[torch.Tensor] = None,
+                                 keep_logits_rows: Optional[int] = 16384, loss_mask: Optional[torch.Tensor] = None):
     """(logprob fp32 [T], entropy fp32 [T]) of ``labels`` under softmax(hidden @ weight.T / temperature).
 
     hidden [T,H] and weight [V,H] share a dtype (bf16 or fp32), labels int64 [T].
@@ -64,10 +96,24 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     backward (the fp32 gradient accumulation FSDP2 does with ``reduce_dtype=fp32``);
     without it ``weight.grad`` gets dW cast to the weight dtype, as torch would.
     Leading dimensions of hidden/labels are flattened and restored.
+
+    ``keep_logits_rows``: when a gradient is needed and there are at most this many rows, the forward
+    keeps its raw logits (one copy in the input dtype, released by the backward) so that the backward
+    does not recompute them; ``None`` or more rows: recompute.  ``loss_mask`` (same shape as
+    ``labels``) is a promise that rows where it is zero receive a zero upstream gradient - true
+    of the reference's loss, which multiplies by this mask (policy_trainer.py:259-283): their
+    logits are then not kept and the backward runs on the other rows only.
     """
     lead = labels.shape
     h2 = hidden.reshape(-1, hidden.shape[-1])
-    lp, ent = _FusedHead.apply(h2, weight, labels.reshape(-1), float(temperature), bool(need_entropy), dweight_buffer)
+    T = h2.shape[0]
+    needs_grad = torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad)
+    keep = bool(needs_grad and keep_logits_rows is not None and T <= keep_logits_rows)
+    mask = None
+    if keep and loss_mask is not None:
+        mask = loss_mask.reshape(-1).to(torch.int32)
+    lp, ent = _FusedHead.apply(h2, weight, labels.reshape(-1), float(temperature), bool(need_entropy), dweight_buffer,
+                               keep, mask)
     lp = lp.reshape(lead)
     ent = ent.reshape(lead) if need_entropy else None
     return lp, ent

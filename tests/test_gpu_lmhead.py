@@ -121,6 +121,52 @@ def test_autograd_function_matches_oracle_autograd(dev):
     assert_close_rel(w.grad, rdw, 1e-5, "weight.grad")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_autograd_kept_logits_mask_hint_and_second_backward(dev, dtype):
+    """The seam keeps its logits for the backward by default; with the loss mask as a hint it keeps
+    and back-propagates only the unmasked rows.  Both must give the gradients of the recomputing
+    path, and a second backward through a retained graph (logits already consumed) must too."""
+    from chatlearn_amd import fused_linear_logprob_entropy
+    T, H, V = 300, 128, 2100
+    hidden, weight, labels = _inputs(T, H, V, dtype, seed=13)
+    g = torch.Generator().manual_seed(3)
+    mask = (torch.rand(T, generator=g) < 0.6).to(torch.int32)
+    c_lp = torch.randn(T, generator=g) * mask
+    c_ent = torch.randn(T, generator=g) * 0.1 * mask
+
+    def grads(retain=False, **kw):
+        h = hidden.to(dev).requires_grad_(True)
+        w = weight.to(dev).requires_grad_(True)
+        lp, ent = fused_linear_logprob_entropy(h, w, labels.to(dev), temperature=0.8, **kw)
+        loss = (lp * c_lp.to(dev)).sum() + (ent * c_ent.to(dev)).sum()
+        loss.backward(retain_graph=retain)
+        first = (h.grad.clone(), w.grad.clone())
+        if retain:
+            h.grad = w.grad = None
+            loss.backward()
+            return first, (h.grad, w.grad)
+        return first
+
+    ref_h, ref_w = grads(keep_logits_rows=None)                        # recompute in the backward
+    rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, c_lp, c_ent, 0.8)
+    r = RTOL[dtype]
+    assert_close_rel(ref_h, rdh, r, "recompute dh")
+    for name, kw in (("kept", {}), ("kept + mask hint", dict(loss_mask=mask.to(dev)))):
+        gh, gw = grads(**kw)
+        assert_close_rel(gh, rdh, r, name + " dh")
+        assert_close_rel(gw, rdw, r, name + " dW")
+    (h1, w1), (h2, w2) = grads(retain=True, loss_mask=mask.to(dev))
+    assert_close_rel(h2, rdh, r, "second backward dh")
+    assert_close_rel(w2, rdw, r, "second backward dW")
+    assert (h1[mask.to(dev) == 0] == 0).all()                          # masked rows get exactly zero
+    # no gradient needed: nothing is kept, results identical
+    with torch.no_grad():
+        lp0, _ = fused_linear_logprob_entropy(hidden.to(dev), weight.to(dev), labels.to(dev), temperature=0.8)
+    lp1, _ = fused_linear_logprob_entropy(hidden.to(dev).requires_grad_(True), weight.to(dev), labels.to(dev),
+                                          temperature=0.8)
+    assert torch.equal(lp0, lp1.detach())
+
+
 def test_argument_errors(dev):
     from chatlearn_amd import ops
     from chatlearn_amd._lib import ClgrpoError
