@@ -168,3 +168,28 @@ def test_vocabulary_shards_merge_to_the_unsharded_result_at_full_size(dev, big):
                                       need_dweight=False, vocab_begin=r * per)
         dh += dh_r.float()
     assert_close_rel(dh, dh0.float(), 1e-2, "sum of the shards' dhidden")
+
+
+def test_fp32_plumbing_configuration_at_full_size_within_1e_5(dev):
+    """c1 at its real shape (fp32, H=1024, the full 151936-row vocabulary): forward and backward within
+    the fp32 tolerance of 1e-5 of the float64 oracle.  The oracle's formulas are evaluated on the
+    device here (float64 GEMMs), which the CPU could not do in test time at this vocabulary."""
+    from chatlearn_amd import ops
+    cfg = synthetic.CONFIGS["c1"]
+    gen = synthetic.generator_for(cfg)
+    samples = synthetic.fill_microbatch(cfg, synthetic.sample_population(cfg, gen))
+    cu, mask = synthetic.packed_layout(samples)
+    T = int(cu[-1])
+    hidden, weight, labels = synthetic.make_head_tensors(cfg, T, gen, device=dev, device_generate=True)
+    assert hidden.dtype == torch.float32 and weight.shape == (151936, 1024)
+    g = torch.Generator(device=dev).manual_seed(1)
+    g_lp = torch.randn(T, generator=g, device=dev) * mask.to(dev)
+    g_ent = torch.randn(T, generator=g, device=dev) * 0.1
+    lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, cfg.temperature)
+    dh, dw = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_ent, cfg.temperature)
+    want = osm.fused_head_forward(hidden, weight, labels, cfg.temperature, torch.float64)
+    rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, g_lp, g_ent, cfg.temperature)
+    assert_close_rel(lp, want[0], 1e-5, "logprob")
+    assert_close_rel(ent, want[1], 1e-5, "entropy")
+    assert_close_rel(dh, rdh, 1e-5, "dhidden")
+    assert_close_rel(dw, rdw, 1e-5, "dweight")
