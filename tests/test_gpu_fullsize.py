@@ -193,3 +193,32 @@ def test_fp32_plumbing_configuration_at_full_size_within_1e_5(dev):
     assert_close_rel(ent, want[1], 1e-5, "entropy")
     assert_close_rel(dh, rdh, 1e-5, "dhidden")
     assert_close_rel(dw, rdw, 1e-5, "dweight")
+
+
+def test_headline_shape_forward_backward_against_the_float64_oracle(dev, big):
+    """The Qwen3-8B head in bf16 (H=4096, V=151936) on a 4096-row slice of the micro-batch, forward
+    and both gradients against the oracle's float64 formulas evaluated on the device; kept-logits
+    path with the masked rows compacted away, as the benchmark step runs it."""
+    from chatlearn_amd import ops
+    T = 4096
+    hidden, labels, weight = big["hidden"][:T].contiguous(), big["labels"][:T].contiguous(), big["weight"]
+    mask = big["mask"][:T]
+    g = torch.Generator(device=dev).manual_seed(5)
+    g_lp = torch.randn(T, generator=g, device=dev) * mask
+    g_ent = torch.randn(T, generator=g, device=dev) * 0.05 * mask
+    live = mask.nonzero().flatten()
+    row_map = torch.full((T,), -1, dtype=torch.int32, device=dev)
+    row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=dev)
+    zbuf = ops.saved_logits_buffer(int(live.numel()), CFG.V, torch.bfloat16, dev)
+    lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, 1.0, saved_logits=zbuf, saved_row_map=row_map)
+    pick = lambda x: x[live].contiguous()
+    dh_c, dw = ops.lmhead_backward(pick(hidden), weight, pick(labels), pick(lse), pick(ent), pick(g_lp), pick(g_ent), 1.0,
+                                   saved_logits=zbuf)
+    dh = torch.zeros(T, CFG.H, dtype=torch.float32, device=dev)
+    dh[live] = dh_c.float()
+    want = osm.fused_head_forward(hidden, weight, labels, 1.0, torch.float64)
+    rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, g_lp, g_ent, 1.0)
+    assert_close_rel(lp, want[0], 1e-2, "logprob")
+    assert_close_rel(ent, want[1], 1e-2, "entropy")
+    assert_close_rel(dh, rdh, 1e-2, "dhidden")
+    assert_close_rel(dw, rdw, 1e-2, "dweight")
