@@ -168,6 +168,69 @@ def library_gemms(hidden, weight, reps=5):
             "dhidden = dlogits @ W": timed(lambda: z @ weight), "dW = dlogits^T @ hidden": timed(lambda: z.t() @ hidden)}
 
 
+def glue_stages(cfg, samples, device, reps=20):
+    """The loss / advantage / index kernels of one micro-batch at this workload's shapes: average
+    time per call (events around `reps` back-to-back calls), bytes each call touches by construction,
+    and launches per call.  They move a few MB at most, so launch latency is what they cost."""
+    from chatlearn_amd.algorithm.grpo_utils.advantage_compute import AdvantageComputer
+    from chatlearn_amd.algorithm.grpo_utils.megatron_utils.train_helper import get_batch_packed
+    p = [s["prompt_token_length"] for s in samples]
+    r = [s["response_token_length"] for s in samples]
+    B, S = len(samples), max(a + b for a, b in zip(p, r))
+    T = sum(p) + sum(r)
+    gen = torch.Generator(device=device).manual_seed(7)
+    tokens = torch.randint(0, cfg.V, (B, S), generator=gen, device=device)
+    plen = torch.tensor(p, dtype=torch.int32, device=device)
+    rlen = torch.tensor(r, dtype=torch.int32, device=device)
+    cu, mask = synthetic.packed_layout(samples)
+    cu, mask = cu.to(device), mask.to(device)
+    lp = -torch.rand(T, generator=gen, device=device)
+    old = lp + 0.01 * torch.randn(T, generator=gen, device=device)
+    ent = torch.rand(T, generator=gen, device=device)
+    adv = torch.randn(B, generator=gen, device=device)
+    attn, lmask, _ = ops.build_masks(plen, rlen, S)
+    idx, *_ = ops.unpad_indices(attn)
+    vec = torch.randn(T, 1, generator=gen, device=device)
+
+    class _Buf:
+        def __init__(self, b):
+            self.buffer = b
+    pop = synthetic.sample_population(cfg, synthetic.generator_for(cfg))
+
+    def advantages():
+        AdvantageComputer(num_inference_per_prompt=cfg.group)([_Buf([dict(x) for x in pop])])
+    stages = {
+        # name: (callable, bytes touched, launches)
+        "build_masks [B,S]": (lambda: ops.build_masks(plen, rlen, S), B * S * 16 + B * 8, 1),
+        "shift_labels [B,S]": (lambda: ops.shift_labels(tokens, lmask, zero_last=True), B * S * 24, 1),
+        "thd_pack (align 1)": (lambda: ops.thd_pack(tokens, p, r, align=1, pad_token=0, want_position_ids=True,
+                                                    verify_on_device=False), T * 44 + B * 20, 2),
+        "pad_input (scatter rows) [T]->[B,S]": (lambda: ops.scatter_rows(vec, idx, B * S), T * 12 + B * S * 4, 2),
+        "policy_loss grpo, upstream grads": (
+            lambda: ops.policy_loss(lp, old, adv, mode=0, cu_seqlens=cu, ref_logprob=old, entropy=ent, loss_mask=mask,
+                                    kl_coef=1e-3, entropy_coef=1e-3, grad_scale=1.0 / T, want_dloss=False,
+                                    want_upstream=True), T * 44, 3),
+        "group advantages (whole episode, host grouping + kernel)": (advantages, len(pop) * 24, 1),
+    }
+    out = {}
+    for name, (fn, nbytes, launches) in stages.items():
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / reps
+        out[name] = {"us_per_call_device_span": e0.elapsed_time(e1) * 1e3 / reps, "us_per_call_wall": wall * 1e6,
+                     "bytes": nbytes, "launches": launches,
+                     "GB_per_s_vs_8000": nbytes / max(e0.elapsed_time(e1) * 1e-3 / reps, 1e-9) / 1e9}
+    return {"B": B, "S": S, "T": T, "episode_samples": len(pop), "stages": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -179,6 +242,8 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=256)
     ap.add_argument("--gemm-reference", action="store_true",
                     help="also time the vendor library's plain GEMMs (torch.matmul) at this head shape, for context")
+    ap.add_argument("--glue", action="store_true",
+                    help="also time the loss / advantage / index kernels at this workload's shapes")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies (a kernel of known HBM traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -334,6 +399,8 @@ def main():
             out["unfused_torch_gpu"] = {"error": str(e)[:200]}
     if args.gemm_reference:
         out["library_gemm_reference"] = library_gemms(hidden, weight)
+    if args.glue:
+        out["glue_stages"] = glue_stages(cfg, samples, dev)
     if not args.no_cpu_baseline:
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
         tps, reps = cpu_baseline(cfg, args.cpu_rows, threads)

@@ -20,6 +20,16 @@ from . import ops
 from ._lib import LOSS_GRPO, LOSS_GSPO
 
 
+def _nonzero_rows(mask: torch.Tensor) -> torch.Tensor:
+    """Ascending positions of the nonzero entries of a flat int32 mask.  The index kernels use one
+    workgroup per row of a [B, S] mask, so the flat mask is presented as many short rows where its
+    length allows (the flat positions are the same)."""
+    n = mask.numel()
+    width = next((w for w in (256, 128, 64) if n % w == 0), n)
+    live, _, _, _ = ops.unpad_indices(mask.reshape(n // width, width))
+    return live
+
+
 class _FusedHead(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, temperature, need_entropy, dweight_buffer, keep_logits, row_mask):
@@ -29,7 +39,7 @@ class _FusedHead(torch.autograd.Function):
             if row_mask is not None:
                 # rows outside the mask get a zero upstream gradient whatever their logits are:
                 # keep logits only for the others and run the backward on that compact set
-                live, _, _, _ = ops.unpad_indices(row_mask.reshape(1, T))
+                live = _nonzero_rows(row_mask)
                 row_map = torch.full((T,), -1, dtype=torch.int32, device=hidden.device)
                 row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
             rows = T if live is None else int(live.numel())
@@ -225,7 +235,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
         if zbuf is not None and loss_mask is not None and skip_masked_rows:
             # Rows whose loss mask is zero get a zero upstream gradient whatever the logits are:
             # keep logits only for the others and run the backward on that compact set of rows.
-            live, _, _, _ = ops.unpad_indices(loss_mask[sl].reshape(1, n))
+            live = _nonzero_rows(loss_mask[sl])
             row_map = torch.full((n,), -1, dtype=torch.int32, device=hidden.device)
             row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
         hook("forward")
