@@ -43,9 +43,9 @@ struct DzParams {
   const float* g_lp;
   const float* g_ent;     // or nullptr
   int Tc;       // valid tokens in the chunk
-  int ldt;      // dzT row stride = Tc rounded up to 64
+  int ldt;      // K extent of dzT = Tc rounded up to 64
   int H, V;
-  int ldv;      // dz row stride = V rounded up to 64
+  int ldv;      // K extent of dz = V rounded up to 64
   int n_tb, n_vt;
   float c, inv_temperature;
   void* dz;     // Tc x ldv, K-blocked (see blocked_index)
