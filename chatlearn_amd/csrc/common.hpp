@@ -11,6 +11,8 @@ namespace clgrpo {
 char* error_buffer();            // thread-local, 512 bytes
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
+// Raises the kernel's dynamic-LDS limit to `bytes` on the current device, once per (kernel, device).
+int ensure_dynamic_lds(const void* kernel, int bytes, const char* name);
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 inline int64_t round_up64(int64_t x, int64_t a) { return (x + a - 1) / a * a; }

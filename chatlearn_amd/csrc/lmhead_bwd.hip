@@ -430,14 +430,6 @@ static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, s
   return lo * 256;
 }
 
-template <typename T>
-static int set_lds_attr(const void* fn, const char* name) {
-  using Tile = HeadTile<T>;
-  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
-  if (e != hipSuccess) return fail(CLGRPO_ELAUNCH, "%s: LDS attribute: %s", name, hipGetErrorString(e));
-  return CLGRPO_OK;
-}
-
 // K ranges per tile that fill the 256 CUs best (1 = no split); at most what `partial_bytes` can hold.
 static int pick_k_split(int tiles, int M, int N, int K, int slab, size_t partial_bytes) {
   int best = 1;
@@ -456,12 +448,8 @@ static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, in
                        int64_t ldc, int accumulate, hipStream_t stream, float* partial = nullptr,
                        size_t partial_bytes = 0) {
   using Tile = HeadTile<T>;
-  static bool attr = false;
-  if (!attr) {
-    int rc = set_lds_attr<T>(reinterpret_cast<const void*>(&gemm_nt_kernel<T, OutT>), "gemm_nt_kernel");
-    if (rc) return rc;
-    attr = true;
-  }
+  int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<T, OutT>), Tile::kLdsBytes, "gemm_nt_kernel");
+  if (rc) return rc;
   GemmParams g;
   g.A = A; g.B = B; g.C = C; g.a_kslabs = a_kslabs; g.b_kslabs = b_kslabs; g.ldc = ldc;
   g.M = M; g.N = N; g.K = K;
@@ -480,7 +468,7 @@ static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, in
   }
   int grid = ((g.n_walk > 0 ? g.n_walk * g.n_nt : g.n_mt * g.n_nt * g.k_split) + 7) / 8 * 8;
   hipLaunchKernelGGL((gemm_nt_kernel<T, OutT>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, g);
-  int rc = check_launch("gemm_nt_kernel");
+  rc = check_launch("gemm_nt_kernel");
   if (rc || g.k_split == 1) return rc;
   const int64_t MN = (int64_t)M * N;
   int blocks = (int)((MN + 255) / 256 < 4096 ? (MN + 255) / 256 : 4096);
@@ -515,13 +503,8 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream, int64_t 
   const T* hidden = static_cast<const T*>(a->hidden);
   const T* weight = static_cast<const T*>(a->weight);
 
-  static bool attr = false;
-  if (!attr) {
-    int rc = set_lds_attr<T>(reinterpret_cast<const void*>(&lmhead_dz_kernel<T>), "lmhead_dz_kernel");
-    if (rc) return rc;
-    attr = true;
-  }
-  int rc;
+  int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&lmhead_dz_kernel<T>), Tile::kLdsBytes, "lmhead_dz_kernel");
+  if (rc) return rc;
   if (a->dhidden && !(a->weight_t && a->weight_t_ready)) {
     // WT(h, v) = W[v][h], zero for V <= v < ldv, K-blocked
     rc = launch_transpose<T>(weight, H, wt, pl.ldv, (int)V, (int)H, stream);

@@ -367,17 +367,12 @@ static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream, int64
   // the K loop's two stages, or the logits tile when it is turned through LDS
   constexpr int kZTile = (STORE_Z && sizeof(T) == 2) ? kFwdBN * kZRow : 0;
   constexpr int lds_bytes = Tile::kLdsBytes > kZTile ? Tile::kLdsBytes : kZTile;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&lmhead_fwd_kernel<T, STORE_Z>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(CLGRPO_ELAUNCH, "lmhead_fwd: LDS attribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&lmhead_fwd_kernel<T, STORE_Z>), lds_bytes, "lmhead_fwd_kernel");
+  if (rc) return rc;
   int grid = p.n_tb * p.n_split;
   grid = (grid + 7) / 8 * 8;
   hipLaunchKernelGGL((lmhead_fwd_kernel<T, STORE_Z>), dim3(grid), dim3(Tile::kThreads), lds_bytes, stream, p);
-  int rc = check_launch("lmhead_fwd_kernel");
+  rc = check_launch("lmhead_fwd_kernel");
   if (rc) return rc;
   FinalizeParams f;
   f.part = p.part;
