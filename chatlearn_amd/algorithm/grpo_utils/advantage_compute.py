@@ -59,21 +59,17 @@ class AdvantageComputer:
             rewards, group_of, torch.tensor(pool, dtype=torch.float64).to(dev),
             torch.tensor(offsets, dtype=torch.int32).to(dev), eps=1e-5)
         adv = adv.cpu().numpy()
-        all_wrong_list = all_zero.cpu().tolist()
-        all_correct_list = all_one.cpu().tolist()
         for s, a in zip(buffers, adv):
             s['advantages'] = a  # numpy.float64, as in the reference
 
-        self.rule_reward_buffer = defaultdict(
-            list, {k: v for k, v in self.rule_reward_buffer.items() if len(v) < self.num_inference_per_prompt})
-        all_correct_ratio = sum(all_correct_list) / len(all_correct_list)
-        all_wrong_ratio = sum(all_wrong_list) / len(all_wrong_list)
-        self._metric_list.append({"all_correct_ratio": all_correct_ratio, "all_wrong_ratio": all_wrong_ratio})
+        # groups that have all their responses are dropped from the pool (advantage_compute.py:40-41)
+        kept = {uid: pool_ for uid, pool_ in self.rule_reward_buffer.items() if len(pool_) < self.num_inference_per_prompt}
+        self.rule_reward_buffer = defaultdict(list, kept)
+        n = float(len(buffers))
+        self._metric_list.append({"all_correct_ratio": int(all_one.sum().item()) / n,
+                                  "all_wrong_ratio": int(all_zero.sum().item()) / n})
         return buffers
 
     def get_and_clear_metrics(self):
-        if self._metric_list is None or len(self._metric_list) == 0:
-            return self._metric_prefix, {}
-        reduced_metrics = _mean_per_key(self._metric_list)
-        self._metric_list = []
-        return self._metric_prefix, reduced_metrics
+        pending, self._metric_list = (self._metric_list or []), []
+        return self._metric_prefix, (_mean_per_key(pending) if pending else {})
