@@ -4,10 +4,8 @@ gathers run in HIP kernels; list regrouping and right-padding of per-sample
 tensors are host-side data marshalling, as in the reference."""
 from collections import defaultdict
 from typing import List, Any, Dict, Optional
-import math
 
 import torch
-import torch.nn.functional as F
 
 from ... import ops
 from ...bert_padding import index_first_axis
@@ -95,15 +93,15 @@ def generate_loss_mask_position_ids(
     attn_mask, loss_mask, position_ids = ops.build_masks(plen, rlen, seq_len, want_position_ids=not prompt_position_ids)
     attn_mask, loss_mask = attn_mask.to(tokens.device), loss_mask.to(tokens.device)
     if prompt_position_ids:
-        # vision-language rows: three position channels given as Python lists; list -> tensor assembly
+        # vision-language rows (reference trainer_utils.py:76-92): three position channels arrive as
+        # Python lists; each is copied in and continued by counting up from its largest value
         position_ids = torch.zeros((3, batch_size, seq_len), dtype=torch.long, device=tokens.device)
-        for batch_idx, batch in enumerate(prompt_position_ids):
-            for list_idx in range(3):
-                sublist = batch[list_idx]
-                position_ids[list_idx, batch_idx, :len(sublist)] = torch.tensor(sublist)
-                start_value = max(sublist) + 1
-                position_ids[list_idx, batch_idx, len(sublist):] = torch.arange(
-                    start_value, start_value + (seq_len - len(sublist)))
+        for b, channels in enumerate(prompt_position_ids):
+            for ch in range(3):
+                given = torch.as_tensor(channels[ch], dtype=torch.long)
+                n = given.numel()
+                position_ids[ch, b, :n] = given
+                position_ids[ch, b, n:] = int(given.max()) + 1 + torch.arange(seq_len - n)
     else:
         position_ids = position_ids.to(tokens.device)
     return attn_mask, loss_mask, position_ids
@@ -116,38 +114,49 @@ def split_microbatch(
     process_group_list: List[Any] = None,
     offset: int = 0, packing: bool = False
 ):
+    """Micro-batches of a mini-batch: token-budget bins when packing, else consecutive runs of
+    ``micro_batch_size`` samples; every sample is tagged with its position ``id_in_list``
+    (reference trainer_utils.py:98-119)."""
     assert micro_batch_size is not None or max_train_token is not None, \
         "At least one of micro_batch_size or max_train_token should be specified"
     if packing:
         return regroup_data_packing(data_list, process_group_list, max_train_token, offset)
-    mini_batch_size = len(data_list)
-    num_micro_batch = math.ceil(mini_batch_size / micro_batch_size)
-    micro_batches = [[] for _ in range(num_micro_batch)]
-    for i in range(num_micro_batch):
-        for sample_id in range(i * micro_batch_size, min((i + 1) * micro_batch_size, mini_batch_size)):
-            data_list[sample_id].update({'id_in_list': sample_id})
-            micro_batches[i].append(data_list[sample_id])
-    return micro_batches
+    total = len(data_list)
+    out = []
+    for start in range(0, total, micro_batch_size):
+        run = []
+        for position in range(start, min(start + micro_batch_size, total)):
+            data_list[position].update({'id_in_list': position})
+            run.append(data_list[position])
+        out.append(run)
+    return out
 
 
 def padding_tensor(tensor_list):
-    dim_size = len(tensor_list[0].shape)
-    seqlen = max(tensor.shape[0] for tensor in tensor_list)
-    return torch.stack([
-        F.pad(t, (0, 0) * (dim_size - 1) + (0, seqlen - t.shape[0])) for t in tensor_list
-    ])
+    """Stack tensors of different first-dimension lengths, zero-padded at the end of that dimension
+    (reference trainer_utils.py:121-129)."""
+    longest = max(t.shape[0] for t in tensor_list)
+    padded = []
+    for t in tensor_list:
+        grown = t.new_zeros((longest,) + tuple(t.shape[1:]))
+        grown[:t.shape[0]] = t
+        padded.append(grown)
+    return torch.stack(padded)
 
 
 def batching(data_list: List[Dict[str, Any]]) -> Dict[str, Any]:
+    """Per-key lists of a micro-batch; tensors are padded and stacked, the two vision keys are
+    concatenated (reference trainer_utils.py:131-146)."""
     if len(data_list) == 0:
         return None
     batched_data = defaultdict(list)
     for key in data_list[0]:
-        batched_data[key] = [data[key] for data in data_list]
-        if key in ['pixel_values', 'image_grid_thw']:
-            batched_data[key] = torch.cat(batched_data[key], dim=0)
-        elif isinstance(batched_data[key][0], torch.Tensor):
-            batched_data[key] = padding_tensor(batched_data[key])
+        column = [sample[key] for sample in data_list]
+        if key in ('pixel_values', 'image_grid_thw'):
+            column = torch.cat(column, dim=0)
+        elif isinstance(column[0], torch.Tensor):
+            column = padding_tensor(column)
+        batched_data[key] = column
     return batched_data
 
 
