@@ -231,6 +231,35 @@ def glue_stages(cfg, samples, device, reps=20):
     return {"B": B, "S": S, "T": T, "episode_samples": len(pop), "stages": out}
 
 
+def autograd_seam(cfg, hidden, weight, labels, mask, steps):
+    """The drop-in seam through torch autograd at this workload's shapes: forward, a linear stand-in
+    for the loss, ``.backward()`` into ``hidden.grad`` and an fp32 main-grad buffer; with the logits
+    recomputed in the backward, kept, and kept with the loss mask as a hint."""
+    from chatlearn_amd import fused_linear_logprob_entropy
+    T = hidden.shape[0]
+    coef = torch.randn(T, device=hidden.device) * mask
+    main_grad = torch.zeros(cfg.V, cfg.H, dtype=torch.float32, device=hidden.device)
+
+    def step(**kw):
+        h = hidden.detach().requires_grad_(True)
+        w = weight.detach().requires_grad_(True)
+        lp, _ = fused_linear_logprob_entropy(h, w, labels, temperature=cfg.temperature, dweight_buffer=main_grad, **kw)
+        ((lp * coef).sum() / T).backward()
+    out = {}
+    for name, kw in (("recompute", dict(keep_logits_rows=None)), ("kept_logits", {}),
+                     ("kept_logits_mask_hint", dict(loss_mask=mask))):
+        for _ in range(2):
+            step(**kw)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(**kw)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        out[name] = {"ms_per_step": dt * 1e3, "tokens_per_s": T / dt}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -242,6 +271,8 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=256)
     ap.add_argument("--gemm-reference", action="store_true",
                     help="also time the vendor library's plain GEMMs (torch.matmul) at this head shape, for context")
+    ap.add_argument("--autograd-seam", action="store_true",
+                    help="also time fused_linear_logprob_entropy through torch autograd (<= 16384 tokens)")
     ap.add_argument("--glue", action="store_true",
                     help="also time the loss / advantage / index kernels at this workload's shapes")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -401,6 +432,8 @@ def main():
         out["library_gemm_reference"] = library_gemms(hidden, weight)
     if args.glue:
         out["glue_stages"] = glue_stages(cfg, samples, dev)
+    if args.autograd_seam and train:
+        out["autograd_seam"] = autograd_seam(cfg, hidden, weight, labels, mask, max(2, args.steps // 2))
     if not args.no_cpu_baseline:
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
         tps, reps = cpu_baseline(cfg, args.cpu_rows, threads)
