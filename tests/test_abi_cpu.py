@@ -87,3 +87,23 @@ def test_cpu_tensors_are_refused():
         ops.lmhead_forward(torch.zeros(2, 64), torch.zeros(4, 64), None)
     with pytest.raises(RuntimeError, match="no CPU path"):
         ops.softmax_stats(torch.zeros(2, 64), None)
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    """No fallback: with the shared object absent the first call that needs it raises and names the
+    build command (checked in a fresh interpreter so the loaded library of this process stays)."""
+    import subprocess
+    import sys
+    code = (
+        "import os, torch\n"
+        f"os.environ['CLGRPO_LIB_PATH'] = {str(tmp_path / 'nowhere.so')!r}\n"
+        "from chatlearn_amd import ops\n"
+        "try:\n"
+        "    ops.bin_packing_ids([3, 2, 1], 4)\n"
+        "except RuntimeError as e:\n"
+        "    assert 'python -m chatlearn_amd.build' in str(e) and 'no fallback' in str(e), str(e)\n"
+        "    print('raised')\n"
+    )
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], cwd=repo, capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "raised" in out.stdout, out.stderr[-500:]
