@@ -9,6 +9,11 @@ Reference semantics restated here (sp_size = 1, fsdp_size = 1, no vision inputs)
 
 ``model(input_ids, position_ids)`` stands for ``self.model(...).logits``: it returns
 logits [b, s, V].  Everything runs on the CPU with the other oracle modules.
+
+Pinned by tests/test_policy_loop_cpu.py: a three-sample case worked by hand from the
+reference lines above (micro-batch order with a tie on the bin totals, packed token row,
+indices, position ids, labels that roll across sequence boundaries, shifted training mask,
+N, per-sample record lengths and values, train_stats) with literal expected tables.
 """
 import torch
 import torch.nn.functional as F
@@ -43,14 +48,12 @@ def preprocess_data_list(data_list, training, *, packing, max_token_in_seq=None,
             pos, *_ = oi.unpad_input(pos.unsqueeze(-1), attn)
             pos = pos.permute(1, 0)
         tokens = tokens_
-        labels = torch.roll(tokens, shifts=-1, dims=1)
+        labels = oi.shift_labels(tokens)
         obj = {"all_tokens": tokens, "position_ids": pos, "labels": labels, "ori_seq_len": ori_len,
                "indices": indices, "ori_batch_size": ori_bs, "sample_ids": b["id_in_list"],
                "attention_mask": attn, "pad_size": 0}
         if training:
-            lm = torch.roll(loss_mask, shifts=-1, dims=1)
-            lm[:, -1] = 0
-            obj.update({"loss_mask": lm, "old_logprobs": b["old_logprobs"], "ref_logprobs": b["ref_logprobs"],
+            obj.update({"loss_mask": oi.shift_loss_mask_fsdp(loss_mask), "old_logprobs": b["old_logprobs"], "ref_logprobs": b["ref_logprobs"],
                         "advantages": b["advantages"]})
         out.append(obj)
     return total_resp, out

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import softmax_stats as osm
-from tests.util import assert_close_rel
+from tests.util import assert_close_rel, assert_contract, assert_rows_rel_l2
 
 pytestmark = pytest.mark.gpu
 
@@ -46,6 +46,9 @@ def test_forward_matches_oracle(dev, T, H, V, dtype, temp):
     assert_close_rel(ent, rent, r, "entropy")
     assert_close_rel(lse, rlse, r, "lse")
     assert_close_rel(mx, rmx, r, "rowmax")
+    # the contract's elementwise form |err| <= atol + rtol |ref|, atol = rtol median|ref|, on every entry
+    assert_contract(lp, rlp, r, "logprob")
+    assert_contract(ent, rent, r, "entropy")
     assert (lp <= 1e-6).all() and (ent >= -1e-6).all() and (ent <= math.log(V) + 1e-4).all()
 
 
@@ -66,6 +69,11 @@ def test_backward_matches_oracle(dev, T, H, V, dtype, temp, with_entropy):
     assert dh.dtype == dtype and dw.dtype == torch.float32
     assert_close_rel(dh, rdh, r, "dhidden")
     assert_close_rel(dw, rdw, r, "dweight")
+    assert_rows_rel_l2(dh.float(), rdh, r, "dhidden rows")
+    assert_rows_rel_l2(dw, rdw, r, "dweight rows")
+    if dtype == torch.float32:
+        assert_contract(dh, rdh, r, "dhidden")
+        assert_contract(dw, rdw, r, "dweight")
 
 
 def test_backward_chunked_equals_unchunked_and_accumulates(dev):

@@ -66,11 +66,18 @@ def test_gspo_mirror_value_flags_grad(dev, B, S):
     assert got[0].dtype == want[0].dtype
     assert_close_rel(got[0], want[0], 1e-5, "gspo loss")
     assert_close_rel(b.grad, a.grad, 1e-5, "gspo grad")
-    # Flags flip only where the fp32 sequence ratio sits within rounding of a clip bound.
+    # The three flags compare the per-sequence ratio with the clip bounds.  They are exact unless a
+    # sequence's ratio lies within fp32 rounding of a bound, which this case excludes (checked here
+    # in float64), so kernel and oracle must agree on every flag of every token.
+    d64 = (lp.double() - old.double()) * mask
+    ratio64 = torch.exp(d64.sum(1) / (mask.sum(1) + 1e-8))
+    live = mask.sum(1) > 0
+    margin = torch.minimum((ratio64 - (1 + 4e-4)).abs(), (ratio64 - (1 - 3e-4)).abs())[live].min()
+    assert margin > 1e-6, "test case sits on a clip bound; pick another seed"
     for name, g_, w_ in zip(("pos", "neg", "clipped"), got[1:], want[1:]):
         assert g_.dtype == torch.bool and g_.shape == w_.shape
-        diff = (g_.cpu() != w_)
-        assert diff.float().mean() < 0.02, f"{name}: {int(diff.sum())} flags differ"
+        assert torch.equal(g_.cpu(), w_), f"{name}: {int((g_.cpu() != w_).sum())} flags differ"
+    assert want[1].any() and want[2].any() and want[3].any()      # every flag occurs in the case
 
 
 @pytest.mark.parametrize("mode", ["grpo", "gspo"])
@@ -161,4 +168,4 @@ def test_megatron_style_outputs(dev):
     assert s[1].item() == pytest.approx(rep["kl_loss"].item(), rel=1e-4, abs=1e-7)
     assert s[2].item() == pytest.approx(rep["entropy_loss"].item(), rel=1e-5)
     assert int(s[3].item()) == int(n)
-    assert abs(s[6].item() - rep["is_clipped"].item()) <= 2
+    assert s[6].item() == rep["is_clipped"].item()
