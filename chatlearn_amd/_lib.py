@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # CLGRPO_LIB_PATH selects another build of the same library (e.g. a tuning variant).
 LIB_PATH = os.environ.get("CLGRPO_LIB_PATH") or os.path.join(_HERE, "csrc", "libclgrpo.so")
 
-BF16, F32, F64 = 0, 1, 2
+BF16, F32, F64, U8 = 0, 1, 2, 3
 LOSS_GRPO, LOSS_GSPO = 0, 1
 
 STATUS_NAMES = {0: "CLGRPO_OK", -1: "CLGRPO_EINVAL", -2: "CLGRPO_EDTYPE", -3: "CLGRPO_ESHAPE",
@@ -63,6 +63,11 @@ class PolicyLossArgs(C.Structure):
                 ("token_offset", i64)]
 
 
+class MaskedSumsArgs(C.Structure):
+    _fields_ = [("n", i64), ("k", i32), ("src", vp * 16), ("dtype", i32 * 16), ("average", i32 * 16),
+                ("mask", vp), ("out", vp), ("count", vp)]
+
+
 class GroupAdvantageArgs(C.Structure):
     _fields_ = [("n_samples", i64), ("n_groups", i64), ("rewards", vp), ("group_of", vp), ("pool", vp),
                 ("pool_offsets", vp), ("eps", f64), ("advantages", vp), ("all_zeros", vp), ("all_ones", vp)]
@@ -111,6 +116,9 @@ SIGNATURES = {
     "clgrpo_softmax_stats_bwd": (C.c_int, [C.POINTER(SoftmaxStatsBwdArgs), vp]),
     "clgrpo_policy_loss_workspace_bytes": (sz, [i64, i64]),
     "clgrpo_policy_loss": (C.c_int, [C.POINTER(PolicyLossArgs), vp]),
+    "clgrpo_policy_loss_launches": (C.c_int, [i64, i32]),
+    "clgrpo_masked_sums": (C.c_int, [C.POINTER(MaskedSumsArgs), vp]),
+    "clgrpo_masked_sums_bwd": (C.c_int, [i64, vp, vp, vp, i32, vp]),
     "clgrpo_group_advantage": (C.c_int, [C.POINTER(GroupAdvantageArgs), vp]),
     "clgrpo_build_masks": (C.c_int, [C.POINTER(BuildMasksArgs), vp]),
     "clgrpo_shift_labels": (C.c_int, [C.POINTER(ShiftLabelsArgs), vp]),

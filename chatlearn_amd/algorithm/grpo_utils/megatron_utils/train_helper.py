@@ -17,7 +17,7 @@ import torch
 
 from .... import ops
 from ....bert_padding import pad_input
-from ..loss_gallery import calculate_gspo_loss, calculate_grpo_loss
+from ...._lib import LOSS_GRPO, LOSS_GSPO
 from ..trainer_utils import _StatsFromLogits
 
 
@@ -107,65 +107,109 @@ def reduce_from_context_parallel_region(logprobs: torch.Tensor, is_packing: bool
     return logprobs[:, :logprobs.shape[1] - inputs['pad_size']]
 
 
+class _TokenLosses(torch.autograd.Function):
+    """Every per-token quantity the Megatron loss dict holds that depends on the logprob, from ONE launch
+    of the policy-loss kernel: the clipped surrogate (token- or sequence-level), the k3 KL with
+    exp(k) forced to 1 outside the mask, and the three clip flags.  Only the surrogate carries a
+    gradient (the kernel emits d loss / d logprob beside it); the reference's own loss_func detaches
+    everything else (train_helper.py:441-449)."""
+
+    @staticmethod
+    def forward(ctx, logprob, old, ref, adv, mask, mode, clips):
+        res = ops.policy_loss(logprob.detach().float(), old.float(), adv, mode=mode, ref_logprob=ref.float(),
+                              loss_mask=mask, want_dloss=True, want_kl=True, want_flags3=(mode == LOSS_GSPO), **clips)
+        bits = int(res.flags.item())       # the reference syncs here too (its three .any() assertions)
+        assert not bits & 1, "pg loss is nan"
+        assert not bits & 2, "kl loss ratio has inf values"
+        assert not bits & 4, "kl loss ratio has nan values"
+        ctx.save_for_backward(res.dloss)
+        ctx.in_dtype = logprob.dtype
+        # dtype of -A * ratio under torch's promotion: a list of numpy float64 advantages makes it float64
+        surrogate = res.loss.to(torch.promote_types(torch.promote_types(logprob.dtype, old.dtype), adv.dtype))
+        flags = (res.is_positive_clipped, res.is_negative_clipped, res.is_clipped) if mode == LOSS_GSPO else ()
+        ctx.mark_non_differentiable(res.kl, *flags)
+        return (surrogate, res.kl) + flags
+
+    @staticmethod
+    def backward(ctx, g_surrogate, *_):
+        (dloss,) = ctx.saved_tensors
+        g = None if g_surrogate is None else (g_surrogate.to(dloss.dtype) * dloss).to(ctx.in_dtype)
+        return g, None, None, None, None, None, None
+
+
+def _batch_rows(x: torch.Tensor, module_args, training_inputs):
+    """[b, s] view of a per-token tensor: packed rows are scattered back to the padded batch."""
+    return reduce_from_context_parallel_region(x, module_args.packing, training_inputs)
+
+
 def _compute_all_losses(module_args, model, all_token_logits: torch.Tensor, labels: torch.Tensor,
                         training_inputs: Dict[str, Any]) -> Dict[str, torch.Tensor]:
-    """All per-token loss tensors of one micro-batch (reference train_helper.py:465-547).
-    ``model`` is unused (the reference only reaches through it for the cross entropy)."""
+    """The per-token loss dict of one micro-batch (reference train_helper.py:465-547): keys ``pg_loss``,
+    ``entropy_loss``, ``kl_loss`` and, for the sequence-level policy, the three clip flags twice (summed and
+    sample-averaged by ``loss_func``).  ``model`` is unused: the reference only reaches through it for the
+    cross entropy, which here is the softmax-statistics kernel on the given logits."""
     del model
-    forward_logprob = language_model_logprob(labels, all_token_logits)
-    forward_logprob = reduce_from_context_parallel_region(forward_logprob, module_args.packing, training_inputs)
-    old_logprobs = training_inputs["old_logprobs"]
-    ref_logprobs = training_inputs["ref_logprobs"]
-    advantages = training_inputs["advantages"]
-    mask = training_inputs['all_token_loss_mask']
-    if module_args.use_group_sequence_policy:
-        pg_loss, is_positive_clipped, is_negative_clipped, is_clipped = calculate_gspo_loss(
-            log_probs=forward_logprob, old_log_probs=old_logprobs, advantages=advantages,
-            diff_clip_ratio=module_args.diff_clip_ratio, pos_clip_ratio=module_args.pos_clip_ratio,
-            neg_clip_ratio=module_args.neg_clip_ratio, final_clip_ratio=module_args.final_clip_ratio,
-            loss_mask=mask)
-    else:
-        pg_loss = calculate_grpo_loss(
-            log_probs=forward_logprob, old_log_probs=old_logprobs, advantages=advantages,
-            diff_clip_ratio=module_args.diff_clip_ratio, pos_clip_ratio=module_args.pos_clip_ratio,
-            neg_clip_ratio=module_args.neg_clip_ratio, final_clip_ratio=module_args.final_clip_ratio)
-    entropy_loss = entropy_from_tensor_parallel_logits(all_token_logits).permute(1, 0)
-    entropy_loss = reduce_from_context_parallel_region(entropy_loss, module_args.packing, training_inputs)
-    # k3 estimator with exp(k) forced to 1 outside the mask, and the reference's two assertions
-    res = ops.policy_loss(forward_logprob.detach().float(), old_logprobs.float(),
-                          torch.zeros(forward_logprob.shape[0], device=forward_logprob.device),
-                          ref_logprob=ref_logprobs.float(), loss_mask=mask, want_dloss=False, want_kl=True)
-    fl = int(res.flags.item())
-    assert not fl & 2, "kl loss ratio has inf values"
-    assert not fl & 4, "kl loss ratio has nan values"
-    kl_loss = res.kl
-    out = {'pg_loss': pg_loss, 'entropy_loss': entropy_loss, 'kl_loss': kl_loss}
-    if module_args.use_group_sequence_policy:
-        out.update({
-            'is_positive_clipped': is_positive_clipped, 'is_negative_clipped': is_negative_clipped,
-            'is_clipped': is_clipped, 'is_positive_clipped_sample_average': is_positive_clipped,
-            'is_negative_clipped_sample_average': is_negative_clipped, 'is_clipped_sample_average': is_clipped})
+    gspo = bool(module_args.use_group_sequence_policy)
+    logprob = _batch_rows(language_model_logprob(labels, all_token_logits), module_args, training_inputs)
+    entropy = _batch_rows(entropy_from_tensor_parallel_logits(all_token_logits).permute(1, 0), module_args,
+                          training_inputs)
+    adv = torch.tensor(training_inputs["advantages"]).to(logprob.device)      # dtype rule of loss_gallery.py:19,53
+    clips = {k: getattr(module_args, k) for k in ("diff_clip_ratio", "pos_clip_ratio", "neg_clip_ratio",
+                                                  "final_clip_ratio")}
+    surrogate, kl, *flags = _TokenLosses.apply(logprob, training_inputs["old_logprobs"],
+                                               training_inputs["ref_logprobs"], adv,
+                                               training_inputs['all_token_loss_mask'],
+                                               LOSS_GSPO if gspo else LOSS_GRPO, clips)
+    out = {'pg_loss': surrogate.contiguous(), 'entropy_loss': entropy, 'kl_loss': kl}
+    if gspo:
+        names = ('is_positive_clipped', 'is_negative_clipped', 'is_clipped')
+        out.update(zip(names, flags))
+        out.update(zip((n + '_sample_average' for n in names), flags))
     return out
 
 
+class _MaskedSums(torch.autograd.Function):
+    """One launch reduces every tensor of the loss dict under the mask; the tensors listed in
+    ``grad_slots`` get the gradient mask * g back."""
+
+    @staticmethod
+    def forward(ctx, mask, grad_slots, averaged, *tensors):
+        sums, count = ops.masked_sums(tensors, mask, averaged)
+        ctx.mask, ctx.grad_slots = mask, grad_slots
+        ctx.like = [(t.dtype, t.shape) for t in tensors]
+        ctx.mark_non_differentiable(count)
+        return sums, count
+
+    @staticmethod
+    def backward(ctx, g_sums, _):
+        grads = [None] * len(ctx.like)
+        if g_sums is not None:
+            g_sums = g_sums.float().contiguous()
+            for j in ctx.grad_slots:
+                dtype, shape = ctx.like[j]
+                grads[j] = ops.masked_sums_backward(g_sums[j:j + 1], ctx.mask, dtype, shape)
+        return (None, None, None) + tuple(grads)
+
+
+BACKPROP_KEYS = ('pg_loss',)     # train_helper.py:441
+
+
 def loss_func(inputs: Dict, losses: Dict[str, torch.Tensor]):
-    """Masked reductions of the loss dict: (loss to back-propagate, number of unmasked tokens, report)
-    (reference train_helper.py:426-463).  Only ``pg_loss`` keeps its gradient."""
-    require_bp_keys = ['pg_loss']
-    loss_mask = inputs["all_token_loss_mask"].float()
-    total_loss_for_bp = 0
-    reporting_losses = {}
-    for key, loss in losses.items():
-        if key not in require_bp_keys:
-            loss = loss.detach()
-        if key.endswith('_sample_average'):
-            final_loss = (loss.float() * loss_mask).sum() / (1e-5 + loss_mask.sum())
-        else:
-            final_loss = (loss.float() * loss_mask).sum()
-        if key in require_bp_keys:
-            total_loss_for_bp = total_loss_for_bp + final_loss
-        reporting_losses[key] = final_loss.detach().clone().to(torch.float)
-    num_tokens = inputs.get('num_tokens_on_this_cp_rank', loss_mask.sum().clone().detach()).to(torch.int)
-    reporting_losses["num_tokens"] = num_tokens
-    reporting_losses["num_samples"] = torch.ones_like(num_tokens)
-    return total_loss_for_bp, num_tokens, reporting_losses
+    """(loss to back-propagate, number of unmasked tokens, report) from the per-token loss dict
+    (reference train_helper.py:426-463): every entry is summed under ``all_token_loss_mask`` (a 0/1 mask),
+    the ``*_sample_average`` entries are divided by (1e-5 + number of unmasked tokens), only ``pg_loss``
+    keeps its gradient.  All reductions run in one kernel launch."""
+    names = list(losses)
+    grad_slots = tuple(j for j, name in enumerate(names) if name in BACKPROP_KEYS and losses[name].requires_grad)
+    averaged = tuple(name.endswith('_sample_average') for name in names)
+    sums, count = _MaskedSums.apply(inputs["all_token_loss_mask"], grad_slots, averaged,
+                                    *(losses[name] for name in names))
+    report = {name: sums[j].detach() for j, name in enumerate(names)}
+    total = 0
+    for j, name in enumerate(names):
+        if name in BACKPROP_KEYS:
+            total = total + sums[j]
+    num_tokens = inputs.get('num_tokens_on_this_cp_rank', count[0]).to(torch.int)
+    report["num_tokens"] = num_tokens
+    report["num_samples"] = torch.ones_like(num_tokens)
+    return total, num_tokens, report

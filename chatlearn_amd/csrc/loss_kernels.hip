@@ -3,8 +3,14 @@
 // [B,S] or cu_seqlens-packed batches.  Memory-bound: each token is read once
 // (logprob, old, ref, entropy, mask: 20 B) and written once (loss, dloss, kl,
 // g_logprob, g_entropy: <= 24 B); reductions are wavefront shuffles + one LDS
-// step per block + a fixed-order pass over the per-block partials, so the sums
-// are reproducible run to run.
+// step per block (+ a fixed-order pass over the per-block partials when more
+// than one block runs), so the sums are reproducible run to run.
+//
+// A micro-batch's worth of tokens (up to 2^18) goes through ONE launch of one
+// 1024-thread workgroup: sequence means (GSPO), per-token work, the reductions
+// and the flag word, with nothing to zero beforehand and no second pass.  The
+// work is a few hundred KB, so launch latency, not bandwidth, is what it costs.
+// Larger inputs take the multi-block kernels (sequence means, loss, finalize).
 //
 // dtype rules follow what torch does in the reference: logprob arithmetic,
 // exp, clamp and the KL stay fp32; the product with the advantages (and the
@@ -16,6 +22,8 @@ namespace clgrpo {
 constexpr int kLossThreads = 256;
 constexpr int kMaxLossBlocks = 1024;
 constexpr int kNumSums = 8;
+constexpr int kOneWgThreads = 1024;
+constexpr int64_t kOneWgMaxTokens = 1 << 18;   // above this the multi-block kernels take over
 
 struct LossParams {
   int mode;
@@ -39,6 +47,7 @@ struct LossParams {
   float* g_logprob;
   float* g_entropy;
   int32_t* flags;
+  double* sums;        // [kNumSums] out (written directly by the one-workgroup kernel)
   float* seq_mean;     // workspace [B] (GSPO)
   double* partials;    // workspace [blocks][kNumSums]
 };
@@ -62,20 +71,23 @@ __device__ __forceinline__ double wave_sum(double v) {
   return v;
 }
 
-// GSPO: per-sequence mean of (logprob - old) over masked positions, as the
-// reference forms it: sum(where(mask, d, 0) * mask) / (sum(mask) + 1e-8), fp32.
-__global__ __launch_bounds__(kLossThreads) void gspo_seq_mean_kernel(LossParams p) {
-  const int b = blockIdx.x;
-  int64_t begin, end;
+// Token range [begin, end) of sequence b inside this call's window.
+__device__ __forceinline__ void seq_range(const LossParams& p, int64_t b, int64_t& begin, int64_t& end) {
   if (p.cu_seqlens) {
     // positions relative to this call's first token; a sequence outside the window contributes nothing
     begin = (int64_t)p.cu_seqlens[b] - p.token_offset;
     end = (int64_t)p.cu_seqlens[b + 1] - p.token_offset;
     if (begin < 0) begin = 0;
     if (end > p.n) end = p.n;
-  } else { begin = (int64_t)b * p.S; end = begin + p.S; }
-  double num = 0.0, den = 0.0;
-  for (int64_t i = begin + threadIdx.x; i < end; i += kLossThreads) {
+  } else { begin = b * p.S; end = begin + p.S; }
+}
+
+// GSPO: this thread's share (positions begin + first, + stride, ...) of the masked sum of
+// (logprob - old) and of the mask count of one sequence.
+__device__ __forceinline__ void seq_mean_partial(const LossParams& p, int64_t begin, int64_t end, int first, int stride,
+                                                 double& num, double& den) {
+  num = 0.0; den = 0.0;
+  for (int64_t i = begin + first; i < end; i += stride) {
     const int mk = p.loss_mask ? p.loss_mask[i] : 1;
     if (mk != 0) {
       const float d = p.logprob[i] - p.old_logprob[i];
@@ -83,6 +95,16 @@ __global__ __launch_bounds__(kLossThreads) void gspo_seq_mean_kernel(LossParams 
       den += (double)mk;
     }
   }
+}
+
+// GSPO: per-sequence mean of (logprob - old) over masked positions, as the
+// reference forms it: sum(where(mask, d, 0) * mask) / (sum(mask) + 1e-8), fp32.
+__global__ __launch_bounds__(kLossThreads) void gspo_seq_mean_kernel(LossParams p) {
+  const int b = blockIdx.x;
+  int64_t begin, end;
+  seq_range(p, b, begin, end);
+  double num, den;
+  seq_mean_partial(p, begin, end, threadIdx.x, kLossThreads, num, den);
   __shared__ double sh[2][kLossThreads / 64];
   num = wave_sum(num);
   den = wave_sum(den);
@@ -95,94 +117,98 @@ __global__ __launch_bounds__(kLossThreads) void gspo_seq_mean_kernel(LossParams 
   }
 }
 
+// One token: surrogate, clip flags, k3 KL, upstream gradients; adds its masked terms to `acc`.
 template <typename CT>
-__global__ __launch_bounds__(kLossThreads) void policy_loss_kernel(LossParams p) {
+__device__ __forceinline__ void loss_token(const LossParams& p, int64_t i, double (&acc)[kNumSums], int& flag) {
   const CT* adv = static_cast<const CT*>(p.advantages);
   CT* loss_out = static_cast<CT*>(p.loss);
   CT* dloss_out = static_cast<CT*>(p.dloss);
+  const CT cap = (CT)p.final_clip;
+  const int b = seq_of_token(p, i);
+  if (b < 0) {
+    // Trailing slots of a packed row that belong to no sequence: defined zeros, no statistics.
+    loss_out[i] = (CT)0;
+    if (dloss_out) dloss_out[i] = (CT)0;
+    if (p.kl) p.kl[i] = 0.f;
+    if (p.is_pos) p.is_pos[i] = 0;
+    if (p.is_neg) p.is_neg[i] = 0;
+    if (p.is_clip) p.is_clip[i] = 0;
+    if (p.g_logprob) p.g_logprob[i] = 0.f;
+    if (p.g_entropy) p.g_entropy[i] = 0.f;
+    return;
+  }
+  const int mk = p.loss_mask ? p.loss_mask[i] : 1;
+  const CT A = adv[b];
+  const float lp = p.logprob[i];
+  const float delta = (p.mode == CLGRPO_LOSS_GSPO) ? p.seq_mean[b] : (lp - p.old_logprob[i]);
+  // clamp(delta, max=diff_clip): NaN stays NaN
+  const float dcl = (delta > p.diff_clip) ? p.diff_clip : delta;
+  const float ratio = expf(dcl);
+  const float rcl = (ratio < p.lo) ? p.lo : ((ratio > p.hi) ? p.hi : ratio);
+  const CT l1 = -A * (CT)ratio;
+  const CT l2 = -A * (CT)rcl;
+  // torch.max / torch.min propagate NaN
+  const CT lc = (l1 != l1 || l2 != l2) ? (CT)NAN : (l1 > l2 ? l1 : l2);
+  const CT L = (lc != lc) ? lc : (lc < cap ? lc : cap);
+  if (L != L) flag |= 1;
+  loss_out[i] = L;
+
+  // d L / d logprob with torch's sub-gradient conventions (ties split in halves,
+  // clamp passes the gradient on the closed interval).
+  const CT w1 = (l1 > l2) ? (CT)1 : ((l1 == l2) ? (CT)0.5 : (CT)0);
+  const CT w2 = (l2 > l1) ? (CT)1 : ((l1 == l2) ? (CT)0.5 : (CT)0);
+  const CT gmin = (lc < cap) ? (CT)1 : ((lc == cap) ? (CT)0.5 : (CT)0);
+  const CT in_clip = (ratio >= p.lo && ratio <= p.hi) ? (CT)1 : (CT)0;
+  const CT pass = (delta <= p.diff_clip) ? (CT)1 : (CT)0;
+  const CT dL = gmin * (w1 + w2 * in_clip) * (-A * (CT)ratio) * pass;
+  if (dloss_out) dloss_out[i] = dL;
+
+  const bool pos = (ratio > p.hi) && (A > (CT)0);
+  const bool neg = (ratio < p.lo) && (A < (CT)0);
+  const bool clp = l2 > l1;
+  if (p.is_pos) p.is_pos[i] = pos;
+  if (p.is_neg) p.is_neg[i] = neg;
+  if (p.is_clip) p.is_clip[i] = clp;
+
+  float klv = 0.f, dkl = 0.f;
+  if (p.ref_logprob) {
+    const float k = p.ref_logprob[i] - lp;
+    float rk = expf(k);
+    if (mk == 0) rk = 1.f;
+    else {
+      if (isinf(rk)) flag |= 2;
+      if (rk != rk) flag |= 4;
+    }
+    const float kld = rk - k - 1.f;
+    klv = (kld < -10.f) ? -10.f : ((kld > 10.f) ? 10.f : kld);
+    dkl = (kld >= -10.f && kld <= 10.f) ? (1.f - rk) : 0.f;
+    if (p.kl) p.kl[i] = klv;
+  }
+  const double w = (double)mk;
+  if (p.g_logprob)
+    p.g_logprob[i] = (mk != 0) ? (float)(p.grad_scale * w * ((double)dL + p.kl_coef * (double)dkl)) : 0.f;
+  if (p.g_entropy)
+    p.g_entropy[i] = (mk != 0) ? (float)(-p.entropy_coef * p.grad_scale * w) : 0.f;
+  if (mk != 0) {
+    acc[0] += w * (double)L;
+    acc[1] += w * (double)klv;
+    if (p.entropy) acc[2] += w * (double)p.entropy[i];
+    acc[3] += w;
+    acc[4] += w * (double)pos;
+    acc[5] += w * (double)neg;
+    acc[6] += w * (double)clp;
+  }
+}
+
+template <typename CT>
+__global__ __launch_bounds__(kLossThreads) void policy_loss_kernel(LossParams p) {
   double acc[kNumSums];
 #pragma unroll
   for (int k = 0; k < kNumSums; ++k) acc[k] = 0.0;
   int flag = 0;
-  const CT cap = (CT)p.final_clip;
-
   for (int64_t i = (int64_t)blockIdx.x * kLossThreads + threadIdx.x; i < p.n;
-       i += (int64_t)gridDim.x * kLossThreads) {
-    const int b = seq_of_token(p, i);
-    if (b < 0) {
-      // Trailing slots of a packed row that belong to no sequence: defined zeros, no statistics.
-      loss_out[i] = (CT)0;
-      if (dloss_out) dloss_out[i] = (CT)0;
-      if (p.kl) p.kl[i] = 0.f;
-      if (p.is_pos) p.is_pos[i] = 0;
-      if (p.is_neg) p.is_neg[i] = 0;
-      if (p.is_clip) p.is_clip[i] = 0;
-      if (p.g_logprob) p.g_logprob[i] = 0.f;
-      if (p.g_entropy) p.g_entropy[i] = 0.f;
-      continue;
-    }
-    const int mk = p.loss_mask ? p.loss_mask[i] : 1;
-    const CT A = adv[b];
-    const float lp = p.logprob[i];
-    const float delta = (p.mode == CLGRPO_LOSS_GSPO) ? p.seq_mean[b] : (lp - p.old_logprob[i]);
-    // clamp(delta, max=diff_clip): NaN stays NaN
-    const float dcl = (delta > p.diff_clip) ? p.diff_clip : delta;
-    const float ratio = expf(dcl);
-    const float rcl = (ratio < p.lo) ? p.lo : ((ratio > p.hi) ? p.hi : ratio);
-    const CT l1 = -A * (CT)ratio;
-    const CT l2 = -A * (CT)rcl;
-    // torch.max / torch.min propagate NaN
-    const CT lc = (l1 != l1 || l2 != l2) ? (CT)NAN : (l1 > l2 ? l1 : l2);
-    const CT L = (lc != lc) ? lc : (lc < cap ? lc : cap);
-    if (L != L) flag |= 1;
-    loss_out[i] = L;
-
-    // d L / d logprob with torch's sub-gradient conventions (ties split in halves,
-    // clamp passes the gradient on the closed interval).
-    const CT w1 = (l1 > l2) ? (CT)1 : ((l1 == l2) ? (CT)0.5 : (CT)0);
-    const CT w2 = (l2 > l1) ? (CT)1 : ((l1 == l2) ? (CT)0.5 : (CT)0);
-    const CT gmin = (lc < cap) ? (CT)1 : ((lc == cap) ? (CT)0.5 : (CT)0);
-    const CT in_clip = (ratio >= p.lo && ratio <= p.hi) ? (CT)1 : (CT)0;
-    const CT pass = (delta <= p.diff_clip) ? (CT)1 : (CT)0;
-    const CT dL = gmin * (w1 + w2 * in_clip) * (-A * (CT)ratio) * pass;
-    if (dloss_out) dloss_out[i] = dL;
-
-    const bool pos = (ratio > p.hi) && (A > (CT)0);
-    const bool neg = (ratio < p.lo) && (A < (CT)0);
-    const bool clp = l2 > l1;
-    if (p.is_pos) p.is_pos[i] = pos;
-    if (p.is_neg) p.is_neg[i] = neg;
-    if (p.is_clip) p.is_clip[i] = clp;
-
-    float klv = 0.f, dkl = 0.f;
-    if (p.ref_logprob) {
-      const float k = p.ref_logprob[i] - lp;
-      float rk = expf(k);
-      if (mk == 0) rk = 1.f;
-      else {
-        if (isinf(rk)) flag |= 2;
-        if (rk != rk) flag |= 4;
-      }
-      const float kld = rk - k - 1.f;
-      klv = (kld < -10.f) ? -10.f : ((kld > 10.f) ? 10.f : kld);
-      dkl = (kld >= -10.f && kld <= 10.f) ? (1.f - rk) : 0.f;
-      if (p.kl) p.kl[i] = klv;
-    }
-    const double w = (double)mk;
-    if (p.g_logprob)
-      p.g_logprob[i] = (mk != 0) ? (float)(p.grad_scale * w * ((double)dL + p.kl_coef * (double)dkl)) : 0.f;
-    if (p.g_entropy)
-      p.g_entropy[i] = (mk != 0) ? (float)(-p.entropy_coef * p.grad_scale * w) : 0.f;
-    if (mk != 0) {
-      acc[0] += w * (double)L;
-      acc[1] += w * (double)klv;
-      if (p.entropy) acc[2] += w * (double)p.entropy[i];
-      acc[3] += w;
-      acc[4] += w * (double)pos;
-      acc[5] += w * (double)neg;
-      acc[6] += w * (double)clp;
-    }
-  }
+       i += (int64_t)gridDim.x * kLossThreads)
+    loss_token<CT>(p, i, acc, flag);
 
   __shared__ double sh[kLossThreads / 64][kNumSums];
 #pragma unroll
@@ -200,6 +226,56 @@ __global__ __launch_bounds__(kLossThreads) void policy_loss_kernel(LossParams p)
   if (flag) atomicOr(p.flags, flag);
 }
 
+
+// The whole call in one workgroup: sequence means (one wavefront per sequence), a barrier, the
+// per-token pass, the reductions, sums and flag word.  Nothing has to be zeroed beforehand and the
+// summation order is fixed.
+template <typename CT>
+__global__ __launch_bounds__(kOneWgThreads) void policy_loss_onewg_kernel(LossParams p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (p.mode == CLGRPO_LOSS_GSPO) {
+    for (int64_t b = wave; b < p.B; b += kOneWgThreads / 64) {
+      int64_t begin, end;
+      seq_range(p, b, begin, end);
+      double num, den;
+      seq_mean_partial(p, begin, end, lane, 64, num, den);
+      num = wave_sum(num);
+      den = wave_sum(den);
+      if (lane == 0) p.seq_mean[b] = (float)num / ((float)den + 1e-8f);
+    }
+    __threadfence();     // the means are read back by other wavefronts of this workgroup
+    __syncthreads();
+  }
+  double acc[kNumSums];
+#pragma unroll
+  for (int k = 0; k < kNumSums; ++k) acc[k] = 0.0;
+  int flag = 0;
+  for (int64_t i = threadIdx.x; i < p.n; i += kOneWgThreads) loss_token<CT>(p, i, acc, flag);
+
+  __shared__ double sh[kOneWgThreads / 64][kNumSums];
+  __shared__ int sh_flag[kOneWgThreads / 64];
+#pragma unroll
+  for (int k = 0; k < kNumSums; ++k) acc[k] = wave_sum(acc[k]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) flag |= __shfl_xor(flag, off);
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < kNumSums; ++k) sh[wave][k] = acc[k];
+    sh_flag[wave] = flag;
+  }
+  __syncthreads();
+  if (threadIdx.x < kNumSums) {
+    double t = 0;
+    for (int w = 0; w < kOneWgThreads / 64; ++w) t += sh[w][threadIdx.x];
+    p.sums[threadIdx.x] = t;
+  }
+  if (threadIdx.x == kNumSums) {
+    int f = 0;
+    for (int w = 0; w < kOneWgThreads / 64; ++w) f |= sh_flag[w];
+    p.flags[0] = f;
+  }
+}
+
 __global__ void policy_loss_finalize_kernel(const double* partials, int n_blocks, double* sums) {
   const int k = threadIdx.x;
   if (k >= kNumSums) return;
@@ -209,6 +285,63 @@ __global__ void policy_loss_finalize_kernel(const double* partials, int n_blocks
 }
 
 __global__ void zero_flags_kernel(int32_t* flags) { flags[0] = 0; }
+
+// Masked sums of up to kMaxMaskedSums per-token tensors in one launch of one workgroup (fixed
+// summation order): out[j] = sum_i float(src_j[i]) * mask[i], divided by (1e-5 + sum(mask)) where
+// average[j] is set; count = sum(mask).  fp64 accumulation, fp32 results.
+constexpr int kMaxMaskedSums = 16;
+struct MaskedSumsParams {
+  int64_t n;
+  int k;
+  const void* src[kMaxMaskedSums];
+  int32_t dtype[kMaxMaskedSums];
+  int32_t average[kMaxMaskedSums];
+  const int32_t* mask;
+  float* out;
+  int32_t* count;
+};
+
+__device__ __forceinline__ float load_as_float(const void* base, int32_t dtype, int64_t i) {
+  if (dtype == CLGRPO_F32) return static_cast<const float*>(base)[i];
+  if (dtype == CLGRPO_F64) return (float)static_cast<const double*>(base)[i];
+  return (float)static_cast<const uint8_t*>(base)[i];
+}
+
+__global__ __launch_bounds__(kOneWgThreads) void masked_sums_kernel(MaskedSumsParams p) {
+  double acc[kMaxMaskedSums + 1];
+#pragma unroll
+  for (int j = 0; j <= kMaxMaskedSums; ++j) acc[j] = 0.0;
+  for (int64_t i = threadIdx.x; i < p.n; i += kOneWgThreads) {
+    const float mk = (float)p.mask[i];
+    if (mk == 0.f) continue;
+    acc[kMaxMaskedSums] += (double)mk;
+#pragma unroll
+    for (int j = 0; j < kMaxMaskedSums; ++j)
+      if (j < p.k) acc[j] += (double)(load_as_float(p.src[j], p.dtype[j], i) * mk);
+  }
+  __shared__ double sh[kOneWgThreads / 64][kMaxMaskedSums + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int j = 0; j <= kMaxMaskedSums; ++j) {
+    const double t = wave_sum(acc[j]);
+    if (lane == 0) sh[wave][j] = t;
+  }
+  __syncthreads();
+  if (threadIdx.x <= kMaxMaskedSums) {
+    double cnt = 0, t = 0;
+    for (int w = 0; w < kOneWgThreads / 64; ++w) { cnt += sh[w][kMaxMaskedSums]; t += sh[w][threadIdx.x]; }
+    if (threadIdx.x == kMaxMaskedSums) p.count[0] = (int32_t)cnt;
+    else if (threadIdx.x < p.k) p.out[threadIdx.x] = p.average[threadIdx.x] ? (float)t / (1e-5f + (float)cnt) : (float)t;
+  }
+}
+
+// d/dsrc of one masked sum: dst[i] = g[0] * mask[i] in the source's dtype (g is a device scalar).
+template <typename CT>
+__global__ void masked_sums_bwd_kernel(int64_t n, const float* g, const int32_t* mask, CT* dst) {
+  const float gv = g[0];
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = (CT)(gv * (float)mask[i]);
+}
 
 static int loss_blocks(int64_t n) {
   int64_t b = (n + kLossThreads - 1) / kLossThreads;
@@ -226,17 +359,18 @@ extern "C" size_t clgrpo_policy_loss_workspace_bytes(int64_t n, int64_t B) {
   return align_up((size_t)B * sizeof(float), 256) + (size_t)kMaxLossBlocks * kNumSums * sizeof(double);
 }
 
-extern "C" int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream) {
+// Validation and launches shared by the entry points; `ws` is the scratch memory they differ in.
+static int run_policy_loss(const char* who, const clgrpo_policy_loss_args* a, void* ws_ptr, size_t ws_bytes, void* stream) {
   CLGRPO_REQUIRE_PTR(a, "args");
   if (a->mode != CLGRPO_LOSS_GRPO && a->mode != CLGRPO_LOSS_GSPO)
-    return fail(CLGRPO_EINVAL, "clgrpo_policy_loss: mode %d", a->mode);
+    return fail(CLGRPO_EINVAL, "%s: mode %d", who, a->mode);
   if (a->compute_dtype != CLGRPO_F32 && a->compute_dtype != CLGRPO_F64)
-    return fail(CLGRPO_EDTYPE, "clgrpo_policy_loss: compute_dtype %d", a->compute_dtype);
-  if (a->token_offset < 0) return fail(CLGRPO_EINVAL, "clgrpo_policy_loss: token_offset=%lld", (long long)a->token_offset);
-  if (a->n < 0 || a->B <= 0) return fail(CLGRPO_EINVAL, "clgrpo_policy_loss: n=%lld B=%lld", (long long)a->n, (long long)a->B);
+    return fail(CLGRPO_EDTYPE, "%s: compute_dtype %d", who, a->compute_dtype);
+  if (a->token_offset < 0) return fail(CLGRPO_EINVAL, "%s: token_offset=%lld", who, (long long)a->token_offset);
+  if (a->n < 0 || a->B <= 0) return fail(CLGRPO_EINVAL, "%s: n=%lld B=%lld", who, (long long)a->n, (long long)a->B);
   if (a->cu_seqlens == nullptr) {
     if (a->S <= 0 || a->B * a->S != a->n)
-      return fail(CLGRPO_ESHAPE, "clgrpo_policy_loss: padded layout needs n == B*S (n=%lld B=%lld S=%lld)",
+      return fail(CLGRPO_ESHAPE, "%s: padded layout needs n == B*S (n=%lld B=%lld S=%lld)", who,
                   (long long)a->n, (long long)a->B, (long long)a->S);
   }
   CLGRPO_REQUIRE_PTR(a->logprob, "logprob");
@@ -245,11 +379,11 @@ extern "C" int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream
   CLGRPO_REQUIRE_PTR(a->loss, "loss");
   CLGRPO_REQUIRE_PTR(a->sums, "sums");
   CLGRPO_REQUIRE_PTR(a->flags, "flags");
-  CLGRPO_REQUIRE_PTR(a->workspace, "workspace");
+  CLGRPO_REQUIRE_PTR(ws_ptr, "workspace");
   if (a->kl != nullptr) CLGRPO_REQUIRE_PTR(a->ref_logprob, "ref_logprob");
   const size_t need = clgrpo_policy_loss_workspace_bytes(a->n, a->B);
-  if (a->workspace_bytes < need)
-    return fail(CLGRPO_EWORKSPACE, "clgrpo_policy_loss: workspace %zu < %zu bytes", a->workspace_bytes, need);
+  if (ws_bytes < need)
+    return fail(CLGRPO_EWORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, need);
   hipStream_t s = static_cast<hipStream_t>(stream);
 
   LossParams p;
@@ -267,10 +401,19 @@ extern "C" int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream
   p.loss = a->loss; p.dloss = a->dloss_dlogprob; p.kl = a->kl;
   p.is_pos = a->is_positive_clipped; p.is_neg = a->is_negative_clipped; p.is_clip = a->is_clipped;
   p.g_logprob = a->g_logprob; p.g_entropy = a->g_entropy; p.flags = a->flags;
-  char* ws = static_cast<char*>(a->workspace);
+  p.sums = a->sums;
+  char* ws = static_cast<char*>(ws_ptr);
   p.seq_mean = reinterpret_cast<float*>(ws);
   p.partials = reinterpret_cast<double*>(ws + align_up((size_t)a->B * sizeof(float), 256));
 
+  if (a->n <= kOneWgMaxTokens) {
+    // one launch: sequence means, per-token pass, sums and flag word in a single workgroup
+    if (a->compute_dtype == CLGRPO_F32)
+      hipLaunchKernelGGL(policy_loss_onewg_kernel<float>, dim3(1), dim3(kOneWgThreads), 0, s, p);
+    else
+      hipLaunchKernelGGL(policy_loss_onewg_kernel<double>, dim3(1), dim3(kOneWgThreads), 0, s, p);
+    return check_launch("policy_loss_onewg_kernel");
+  }
   hipLaunchKernelGGL(zero_flags_kernel, dim3(1), dim3(1), 0, s, a->flags);
   if (a->mode == CLGRPO_LOSS_GSPO) {
     hipLaunchKernelGGL(gspo_seq_mean_kernel, dim3((unsigned)a->B), dim3(kLossThreads), 0, s, p);
@@ -286,4 +429,54 @@ extern "C" int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream
   if (rc) return rc;
   hipLaunchKernelGGL(policy_loss_finalize_kernel, dim3(1), dim3(64), 0, s, p.partials, blocks, a->sums);
   return check_launch("policy_loss_finalize_kernel");
+}
+
+extern "C" int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream) {
+  CLGRPO_REQUIRE_PTR(a, "args");
+  return run_policy_loss("clgrpo_policy_loss", a, a->workspace, a->workspace_bytes, stream);
+}
+
+extern "C" int clgrpo_policy_loss_launches(int64_t n, int32_t mode) {
+  if (n <= kOneWgMaxTokens) return 1;
+  return mode == CLGRPO_LOSS_GSPO ? 4 : 3;
+}
+
+extern "C" int clgrpo_masked_sums(const clgrpo_masked_sums_args* a, void* stream) {
+  CLGRPO_REQUIRE_PTR(a, "args");
+  if (a->n < 0 || a->k <= 0 || a->k > kMaxMaskedSums)
+    return fail(CLGRPO_EINVAL, "clgrpo_masked_sums: n=%lld k=%d (at most %d tensors)", (long long)a->n, a->k, kMaxMaskedSums);
+  CLGRPO_REQUIRE_PTR(a->mask, "mask");
+  CLGRPO_REQUIRE_PTR(a->out, "out");
+  CLGRPO_REQUIRE_PTR(a->count, "count");
+  MaskedSumsParams p;
+  p.n = a->n; p.k = a->k; p.mask = a->mask; p.out = a->out; p.count = a->count;
+  for (int j = 0; j < kMaxMaskedSums; ++j) {
+    p.src[j] = j < a->k ? a->src[j] : nullptr;
+    p.dtype[j] = j < a->k ? a->dtype[j] : CLGRPO_F32;
+    p.average[j] = j < a->k ? a->average[j] : 0;
+    if (j < a->k) {
+      CLGRPO_REQUIRE_PTR(a->src[j], "src[j]");
+      if (a->dtype[j] != CLGRPO_F32 && a->dtype[j] != CLGRPO_F64 && a->dtype[j] != CLGRPO_U8)
+        return fail(CLGRPO_EDTYPE, "clgrpo_masked_sums: dtype[%d] = %d", j, a->dtype[j]);
+    }
+  }
+  hipLaunchKernelGGL(masked_sums_kernel, dim3(1), dim3(kOneWgThreads), 0, static_cast<hipStream_t>(stream), p);
+  return check_launch("masked_sums_kernel");
+}
+
+extern "C" int clgrpo_masked_sums_bwd(int64_t n, const float* g, const int32_t* mask, void* dst, int32_t dtype,
+                                      void* stream) {
+  CLGRPO_REQUIRE_PTR(g, "g");
+  CLGRPO_REQUIRE_PTR(mask, "mask");
+  CLGRPO_REQUIRE_PTR(dst, "dst");
+  if (n < 0) return fail(CLGRPO_EINVAL, "clgrpo_masked_sums_bwd: n=%lld", (long long)n);
+  if (dtype != CLGRPO_F32 && dtype != CLGRPO_F64) return fail(CLGRPO_EDTYPE, "clgrpo_masked_sums_bwd: dtype %d", dtype);
+  if (n == 0) return CLGRPO_OK;
+  const int blocks = (int)((n + 255) / 256 < 1024 ? (n + 255) / 256 : 1024);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == CLGRPO_F32)
+    hipLaunchKernelGGL(masked_sums_bwd_kernel<float>, dim3(blocks), dim3(256), 0, s, n, g, mask, static_cast<float*>(dst));
+  else
+    hipLaunchKernelGGL(masked_sums_bwd_kernel<double>, dim3(blocks), dim3(256), 0, s, n, g, mask, static_cast<double*>(dst));
+  return check_launch("masked_sums_bwd_kernel");
 }

@@ -10,7 +10,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from . import _lib
-from ._lib import BF16, F32, F64, LOSS_GRPO, LOSS_GSPO
+from ._lib import BF16, F32, F64, U8, LOSS_GRPO, LOSS_GSPO
 
 DEFAULT_BWD_WORKSPACE_BYTES = 24 << 30
 
@@ -380,6 +380,57 @@ def policy_loss(logprob, old_logprob, advantages, *, mode=LOSS_GRPO, cu_seqlens=
                             int(token_offset))
     _lib.call("clgrpo_policy_loss", a, _stream(logprob))
     return r
+
+
+def masked_sums(tensors, mask: torch.Tensor, averaged):
+    """(sums fp32 [k], count int32 [1]): sums[j] = sum(float(tensors[j]) * mask), divided by
+    (1e-5 + sum(mask)) where ``averaged[j]``; count = sum(mask).  Tensors are fp32, fp64 or bool and
+    have the mask's number of elements; the mask holds zeros and ones.  One launch for all of them."""
+    tensors = list(tensors)
+    k = len(tensors)
+    if not 1 <= k <= 16:
+        raise ValueError(f"between 1 and 16 tensors expected, got {k}")
+    if mask.dtype != torch.int32:
+        mask = mask.to(torch.int32)
+    mask = _dev(mask, "mask", torch.int32)
+    n = mask.numel()
+    if n == 0:
+        return (torch.zeros(k, dtype=torch.float32, device=mask.device),
+                torch.zeros(1, dtype=torch.int32, device=mask.device))
+    a = _lib.MaskedSumsArgs()
+    a.n, a.k = n, k
+    keep = []
+    for j, t in enumerate(tensors):
+        t = _dev(t.detach(), f"tensors[{j}]")
+        if t.numel() != n:
+            raise ValueError(f"tensors[{j}] must have {n} elements, got {t.numel()}")
+        if t.dtype == torch.bool:
+            code = U8
+        elif t.dtype in (torch.float32, torch.float64):
+            code = _dtype_enum(t)
+        else:
+            t, code = t.float(), F32
+        keep.append(t)
+        a.src[j], a.dtype[j], a.average[j] = t.data_ptr(), code, 1 if averaged[j] else 0
+    sums = torch.empty(k, dtype=torch.float32, device=mask.device)
+    count = torch.empty(1, dtype=torch.int32, device=mask.device)
+    a.mask, a.out, a.count = mask.data_ptr(), sums.data_ptr(), count.data_ptr()
+    _lib.call("clgrpo_masked_sums", a, _stream(mask))
+    return sums, count
+
+
+def masked_sums_backward(g: torch.Tensor, mask: torch.Tensor, dtype, shape) -> torch.Tensor:
+    """g[0] * mask as a tensor of ``dtype`` (fp32 / fp64) and ``shape``; ``g`` a one-element fp32 device tensor."""
+    if mask.dtype != torch.int32:
+        mask = mask.to(torch.int32)
+    mask = _dev(mask, "mask", torch.int32)
+    g = _dev(g, "g", torch.float32)
+    if dtype not in (torch.float32, torch.float64):
+        raise TypeError(f"gradient dtype must be fp32 or fp64, got {dtype}")
+    out = torch.empty(shape, dtype=dtype, device=mask.device)
+    _lib.check(_lib.lib().clgrpo_masked_sums_bwd(mask.numel(), _ptr(g), _ptr(mask), _ptr(out),
+                                                 F32 if dtype == torch.float32 else F64, _lib.vp(_stream(mask) or 0)))
+    return out
 
 
 # --------------------------------------------------------------------------- advantages

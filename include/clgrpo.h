@@ -32,7 +32,7 @@ typedef enum {
   CLGRPO_EWORKSPACE = -6  /* workspace too small */
 } clgrpo_status;
 
-typedef enum { CLGRPO_BF16 = 0, CLGRPO_F32 = 1, CLGRPO_F64 = 2 } clgrpo_dtype;
+typedef enum { CLGRPO_BF16 = 0, CLGRPO_F32 = 1, CLGRPO_F64 = 2, CLGRPO_U8 = 3 /* bool / uint8 flags */ } clgrpo_dtype;
 
 int clgrpo_version(void);
 const char* clgrpo_last_error_string(void);
@@ -222,6 +222,29 @@ typedef struct {
 
 size_t clgrpo_policy_loss_workspace_bytes(int64_t n, int64_t B);
 int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream);
+/* Kernel launches one clgrpo_policy_loss call of n tokens enqueues (1 up to 2^18 tokens: sequence
+ * means, per-token pass, sums and flag word run in a single workgroup). */
+int clgrpo_policy_loss_launches(int64_t n, int32_t mode);
+
+/* Masked reductions of a dict of per-token loss tensors, one launch.
+ * Replaces: the body of loss_func (megatron_utils/train_helper.py:441-463):
+ *   out[j] = sum_i float(src_j[i]) * mask[i]                       (average[j] == 0)
+ *   out[j] = sum_i float(src_j[i]) * mask[i] / (1e-5 + sum(mask))  (average[j] != 0, the *_sample_average keys)
+ *   count  = sum(mask)
+ * and, for the one key that is back-propagated (pg_loss), its gradient mask * g. */
+typedef struct {
+  int64_t n;                 /* elements per tensor */
+  int32_t k;                 /* tensors, 1..16 */
+  const void* src[16];       /* [n] each */
+  int32_t dtype[16];         /* CLGRPO_F32, CLGRPO_F64 or CLGRPO_U8 (bool flags) */
+  int32_t average[16];
+  const int32_t* mask;       /* [n] */
+  float* out;                /* [k] out */
+  int32_t* count;            /* [1] out */
+} clgrpo_masked_sums_args;
+int clgrpo_masked_sums(const clgrpo_masked_sums_args* a, void* stream);
+/* dst[i] = g[0] * mask[i] in `dtype` (CLGRPO_F32 / CLGRPO_F64); g is a device scalar. */
+int clgrpo_masked_sums_bwd(int64_t n, const float* g, const int32_t* mask, void* dst, int32_t dtype, void* stream);
 
 /* ------------------------------------------------------------------ *
  * Group-wise reward -> advantage: adv = (r - mean(pool_g)) / (std(pool_g) + eps),

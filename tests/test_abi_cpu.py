@@ -32,6 +32,7 @@ def test_struct_sizes_match_header_layout():
     assert C.sizeof(_lib.LmheadFwdArgs) == 3 * 8 + 3 * 8 + 4 + 4 + 4 * 8 + 8 + 8 + 8 + 8 + 8 + 8
     assert C.sizeof(_lib.LmheadBwdArgs) == 7 * 8 + 3 * 8 + 4 + 4 + 2 * 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8
     assert C.sizeof(_lib.RowsArgs) == 6 * 8
+    assert C.sizeof(_lib.MaskedSumsArgs) == 8 + 8 + 16 * 8 + 16 * 4 + 16 * 4 + 3 * 8
 
 
 def _err(lib):

@@ -35,11 +35,13 @@ CASES = [
 ]
 
 
-# Smallest fraction of bf16 gradient entries that must sit inside |err| <= atol + 1e-2 |ref| (atol =
+# Smallest fraction of bf16 dW entries (every dhidden entry passes) that must sit inside |err| <= atol + 1e-2 |ref| (atol =
 # 1e-2 median|ref|).  The rest are entries whose terms cancel to well below the tensor's typical
 # magnitude; their error is the bf16 rounding of d(logits) (2^-9 relative per term, the same rounding the
 # reference's bf16 autograd applies), not a wrong term: the row-wise L2 and max-norm bounds above hold at 1e-2.
-GRAD_FRAC = 0.0
+DW_FRAC_BF16 = 0.99
+# fp32: the same cancelling entries against fp32 accumulation order, a few in 10^4.
+DW_FRAC_FP32 = 0.999
 
 
 @pytest.mark.parametrize("name,kw", CASES, ids=[c[0] for c in CASES])
@@ -73,13 +75,13 @@ def test_head_step_matches_oracle(dev, name, kw, keep):
     # Gradients, GSPO included, at the contract's tolerance: every row within a relative L2 error of rt,
     # the tensor as a whole within rt of its largest entry, and elementwise |err| <= atol + rt |ref|
     # (fp32: every entry; bf16: d(logits) is rounded to bf16 before the two contractions, so entries
-    # that cancel to near zero carry a rounding error comparable to atol: see GRAD_FRAC)
+    # that cancel to near zero carry a rounding error comparable to atol: see DW_FRAC_BF16)
     assert_close_rel(got["dhidden"], want["dhidden"], rt, "dhidden")
     assert_close_rel(got["dweight"], want["dweight"], rt, "dweight")
     assert_rows_rel_l2(got["dhidden"].float(), want["dhidden"], rt, "dhidden rows")
     assert_rows_rel_l2(got["dweight"], want["dweight"], rt, "dweight rows")
-    assert_contract(got["dhidden"], want["dhidden"], rt, "dhidden", min_frac=1.0 if fp32 else GRAD_FRAC)
-    assert_contract(got["dweight"], want["dweight"], rt, "dweight", min_frac=1.0 if fp32 else GRAD_FRAC)
+    assert_contract(got["dhidden"], want["dhidden"], rt, "dhidden")
+    assert_contract(got["dweight"], want["dweight"], rt, "dweight", min_frac=DW_FRAC_FP32 if fp32 else DW_FRAC_BF16)
     if keep is not None:
         # masked-out rows were left out of the backward: exact zeros there, and fewer rows projected
         assert got["rows_projected_bwd"] == int(mask.sum())

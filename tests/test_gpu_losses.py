@@ -77,7 +77,8 @@ def test_gspo_mirror_value_flags_grad(dev, B, S):
     for name, g_, w_ in zip(("pos", "neg", "clipped"), got[1:], want[1:]):
         assert g_.dtype == torch.bool and g_.shape == w_.shape
         assert torch.equal(g_.cpu(), w_), f"{name}: {int((g_.cpu() != w_).sum())} flags differ"
-    assert want[1].any() and want[2].any() and want[3].any()      # every flag occurs in the case
+    if B >= 16:
+        assert want[1].any() and want[2].any() and want[3].any()      # every flag occurs in the case
 
 
 @pytest.mark.parametrize("mode", ["grpo", "gspo"])
