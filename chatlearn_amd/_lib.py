@@ -117,6 +117,8 @@ SIGNATURES = {
     "clgrpo_policy_loss_workspace_bytes": (sz, [i64, i64]),
     "clgrpo_policy_loss": (C.c_int, [C.POINTER(PolicyLossArgs), vp]),
     "clgrpo_policy_loss_launches": (C.c_int, [i64, i32]),
+    "clgrpo_policy_loss_static": (C.c_int, [C.POINTER(PolicyLossArgs), vp]),
+    "clgrpo_policy_loss_static_max_sequences": (i64, []),
     "clgrpo_masked_sums": (C.c_int, [C.POINTER(MaskedSumsArgs), vp]),
     "clgrpo_masked_sums_bwd": (C.c_int, [i64, vp, vp, vp, i32, vp]),
     "clgrpo_group_advantage": (C.c_int, [C.POINTER(GroupAdvantageArgs), vp]),

@@ -16,6 +16,7 @@
 // exp, clamp and the KL stay fp32; the product with the advantages (and the
 // final cap) is carried in the advantages' dtype, fp32 or fp64.
 #include "common.hpp"
+#include <mutex>
 
 namespace clgrpo {
 
@@ -434,6 +435,51 @@ static int run_policy_loss(const char* who, const clgrpo_policy_loss_args* a, vo
 extern "C" int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream) {
   CLGRPO_REQUIRE_PTR(a, "args");
   return run_policy_loss("clgrpo_policy_loss", a, a->workspace, a->workspace_bytes, stream);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// Scratch memory of clgrpo_policy_loss_static: what the other entry point takes from the caller's
+// workspace (sequence means for up to kStaticMaxSeqs sequences, then the per-block partial sums).
+// Each device the library runs on holds its own copy of this array until the process ends.  Nothing
+// in it has to start at zero: every call writes the means of all its sequences and the partials of
+// all its blocks before reading them.  Calls that overlap on one device share it and race.
+constexpr int64_t kStaticMaxSeqs = 65536;
+constexpr size_t kStaticScratchBytes = (size_t)kStaticMaxSeqs * sizeof(float) + (size_t)kMaxLossBlocks * kNumSums * sizeof(double);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device, looked up once per device (the array's name is
+// only a host-side handle of the symbol, not an address a kernel could use).
+static int static_scratch_address(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* address[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(CLGRPO_ELAUNCH, "clgrpo_policy_loss_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(CLGRPO_EINVAL, "clgrpo_policy_loss_static: device %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (address[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(CLGRPO_ELAUNCH, "clgrpo_policy_loss_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    address[dev] = ptr;
+  }
+  *out = address[dev];
+  return CLGRPO_OK;
+}
+
+extern "C" int64_t clgrpo_policy_loss_static_max_sequences(void) { return kStaticMaxSeqs; }
+
+extern "C" int clgrpo_policy_loss_static(const clgrpo_policy_loss_args* a, void* stream) {
+  CLGRPO_REQUIRE_PTR(a, "args");
+  if (a->B > kStaticMaxSeqs)
+    return fail(CLGRPO_EWORKSPACE, "clgrpo_policy_loss_static: B=%lld sequences exceed the built-in scratch (at most %lld); "
+                "use clgrpo_policy_loss with a workspace", (long long)a->B, (long long)kStaticMaxSeqs);
+  void* ptr = nullptr;
+  int rc = static_scratch_address(&ptr);
+  if (rc) return rc;
+  return run_policy_loss("clgrpo_policy_loss_static", a, ptr, kStaticScratchBytes, stream);
 }
 
 extern "C" int clgrpo_policy_loss_launches(int64_t n, int32_t mode) {

@@ -226,6 +226,17 @@ int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream);
  * means, per-token pass, sums and flag word run in a single workgroup). */
 int clgrpo_policy_loss_launches(int64_t n, int32_t mode);
 
+/* clgrpo_policy_loss without a workspace and without any allocation.  No counterpart in the reference: it
+ * is for callers that cannot allocate device memory around the call (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  Same arguments and results as clgrpo_policy_loss,
+ * bit for bit; `workspace` / `workspace_bytes` are ignored (may be NULL / 0).  The scratch memory is a
+ * 320 KiB array built into the library, one copy per device: at most
+ * clgrpo_policy_loss_static_max_sequences() = 65536 sequences per call (any number of tokens), more is
+ * refused with CLGRPO_EWORKSPACE.  Calls that overlap on one device (two streams) share the array and race:
+ * keep them in stream order, or use clgrpo_policy_loss with separate workspaces. */
+int clgrpo_policy_loss_static(const clgrpo_policy_loss_args* a, void* stream);
+int64_t clgrpo_policy_loss_static_max_sequences(void);
+
 /* Masked reductions of a dict of per-token loss tensors, one launch.
  * Replaces: the body of loss_func (megatron_utils/train_helper.py:441-463):
  *   out[j] = sum_i float(src_j[i]) * mask[i]                       (average[j] == 0)
