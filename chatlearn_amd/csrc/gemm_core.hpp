@@ -55,6 +55,42 @@ __host__ __device__ __forceinline__ int64_t blocked_index(int64_t row, int64_t k
   return (((row / kBlockRows) * n_kslab + k / E) * kBlockRows + (row % kBlockRows)) * E + (k % E);
 }
 
+// Kept logits ("z-native" layout).  The forward leaves a chunk's raw logits for the backward in the
+// order its accumulators hold them, so that storing them costs no shuffle: the buffer is cut into the
+// same 32 KB units as a K-blocked operand (256 rows x one 128-byte K slab of vocabulary, unit (rb, ks) at
+// byte (rb * n_kslab + ks) * 32768), and inside a unit into sub-blocks of 32 rows x 32 vocabulary entries,
+// sub-block (rs, vs) at (rs * VSUB + vs) * PIECES KB.  A sub-block is one 32x32 accumulator block: lane
+// (h, t32) = (lane / 32, lane % 32) owns row t32 and the 16 entries 8 * (r / 4) + 4 * h + r % 4, r = 0..15,
+// which it stores as PIECES 16-byte pieces; piece j of all 64 lanes is one contiguous KB.  The kernel that
+// turns logits into d(logits) reads a unit whole and writes the K-blocked result over it.
+// 16-bit inputs keep their logits as IEEE half (10 mantissa bits against bf16's 7: the softmax the
+// backward rebuilds from them is 8x closer to the fp32 one), fp32 inputs as fp32.
+template <typename T> struct KeptLogit;
+template <> struct KeptLogit<__bf16> { typedef _Float16 type; };
+template <> struct KeptLogit<float> { typedef float type; };
+
+template <typename T> struct ZNative {
+  static constexpr int ES = (int)sizeof(T);
+  static constexpr int kSlabElems = kRowBytes / ES;     // vocabulary entries per unit
+  static constexpr int VSUB = kSlabElems / 32;          // sub-blocks along the vocabulary per unit
+  static constexpr int PIECES = ES;                     // 16-byte pieces per lane and sub-block (16 values)
+  static constexpr int kPerPiece = 16 / PIECES;         // values per piece
+  static constexpr int kUnitBytes = kBlockRows * kRowBytes;
+  // byte offset of piece j of lane half h for `row` and the 32-aligned vocabulary block `v32` (= vocab / 32)
+  __host__ __device__ static __forceinline__ int64_t piece_offset(int64_t row, int64_t v32, int64_t n_kslab, int h, int j) {
+    const int64_t rb = row / kBlockRows;
+    const int R = (int)(row % kBlockRows);
+    const int64_t unit = (rb * n_kslab + v32 / VSUB) * kUnitBytes;
+    const int sb = (R >> 5) * VSUB + (int)(v32 % VSUB);
+    return unit + (int64_t)sb * (PIECES * 1024) + j * 1024 + (h * 32 + (R & 31)) * 16;
+  }
+  // vocabulary offset inside its 32-block of value e of piece j for lane half h
+  __host__ __device__ static __forceinline__ int col_of(int h, int j, int e) {
+    const int r = j * kPerPiece + e;
+    return 8 * (r >> 2) + 4 * h + (r & 3);
+  }
+};
+
 // One 32-byte-of-K step for a 32x32 block: a and b each hold 16 bytes per lane.
 template <typename T>
 __device__ __forceinline__ void mma_block(f32x16& acc, const u32x4& a, const u32x4& b);

@@ -145,14 +145,16 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_dz_kernel(DzParams p) {
   }
 }
 
-// d(logits) from stored logits, in place, plus its transpose.  One 64 x 64 (token x vocabulary)
-// tile per workgroup: read z (16 bytes per lane along the vocabulary), form dz with the per-token
-// coefficients, write it back over z, and turn the tile through LDS so dzT[vocab][token] is also
-// written in 16-byte pieces.  Both are K-blocked operands of the GEMMs that follow, so a tile's
-// 64 rows of 128 bytes are one contiguous 8 KB run on either side.  HBM-bound: reads 1x, writes
-// 2x the chunk.
+// d(logits) from kept logits, in place, plus its transpose.  One workgroup per 32 KB unit of the kept
+// logits (256 token rows x one 128-byte slab of vocabulary, z-native layout, see ZNative): every thread
+// reads its 128 bytes of the unit, forms dz with its rows' coefficients and drops the values into two LDS
+// tiles, [token][vocab] and [vocab][token]; after a barrier the first goes back over the unit as the
+// K-blocked dz operand (the unit's 32 KB are exactly that operand's piece for these rows and this slab)
+// and the second to the K-blocked dzT operand (per 64-token slab one contiguous piece of 64 vocabulary
+// rows).  All global accesses are 16 bytes per lane and contiguous per wavefront.  HBM-bound: reads 1x,
+// writes 2x the chunk.
 struct DzFromZParams {
-  void* z;            // Tc x ldv, K-blocked; in: raw logits, out: dz
+  void* z;            // Tc x ldv: in kept logits (z-native, KeptLogit<T>), out dz (K-blocked, T)
   void* dzT;          // V x ldt, K-blocked
   const int64_t* labels;
   int64_t label_offset;
@@ -166,54 +168,115 @@ struct DzFromZParams {
 
 template <typename T>
 __global__ __launch_bounds__(256) void dz_from_z_kernel(DzFromZParams p) {
-  constexpr int VEC = 16 / (int)sizeof(T);       // elements per 16-byte access
-  constexpr int kE = kRowBytes / (int)sizeof(T); // elements per K slab of a blocked operand
-  constexpr int CPR = 64 / VEC;                  // accesses per 64-wide tile row
-  constexpr int RPP = 256 / CPR;                 // tile rows covered per pass
-  __shared__ T tile[64][64 + VEC];               // [vocab][token], padded rows
-  const int t0 = blockIdx.x * 64, v0 = blockIdx.y * 64;
-  const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
-  T* z = static_cast<T*>(p.z);
-  T* dzT = static_cast<T*>(p.dzT);
+  typedef typename KeptLogit<T>::type ZT;
+  typedef ZNative<ZT> ZL;
+  static_assert(sizeof(ZT) == sizeof(T), "d(logits) overwrites the kept logits in place");
+  constexpr int E = ZL::kSlabElems;                 // vocabulary entries of this unit (64 or 32)
+  constexpr int VEC = 16 / (int)sizeof(T);          // elements per 16-byte piece
+  constexpr int kSub = 8 * ZL::VSUB;                // 32x32 sub-blocks per unit
+  constexpr int kSubPerWave = kSub / 4;
+  constexpr int kTPitch = kBlockRows * (int)sizeof(T) + 16;   // bytes per vocabulary row of the transposed tile
+  // one LDS region, used twice: [token R][vocab c] with the 16-byte chunks XOR-swizzled by R % 8 (32 KB),
+  // then [vocab c][token R] with padded rows
+  __shared__ __align__(16) char tile[E * kTPitch > kBlockRows * kRowBytes ? E * kTPitch : kBlockRows * kRowBytes];
+  const int rb = blockIdx.x, ks = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int h = lane >> 5, t32 = lane & 31;
+  const int64_t n_kslab = p.ldv / E;
+  char* unit = static_cast<char*>(p.z) + ((int64_t)rb * n_kslab + ks) * ZL::kUnitBytes;
   const float it = p.inv_temperature;
-  for (int rr = r; rr < 64; rr += RPP) {
-    const int t = t0 + rr;
-    const int v = v0 + c * VEC;
-    alignas(16) T vals[VEC];
+
+  u32x4 raw[kSubPerWave][ZL::PIECES];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) vals[j] = (T)0.f;
-    if (t < p.Tc && v < p.ldv) {
-      const float glp = p.g_lp[t];
-      const float gen = p.g_ent ? p.g_ent[t] : 0.f;
-      if (glp != 0.f || gen != 0.f) {
-        const float lse = p.lse[t];
-        const float lse2 = lse * kLog2e;
-        const float ent = p.g_ent ? p.entropy[t] : 0.f;
-        const int64_t lab = p.labels[t] - p.label_offset;
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(z + blocked_index<T>(t, v, p.ldv / kE));
-        const T* in = reinterpret_cast<const T*>(&raw);
+  for (int s = 0; s < kSubPerWave; ++s)
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const float zraw = (float)in[j];
+    for (int j = 0; j < ZL::PIECES; ++j)
+      raw[s][j] = *reinterpret_cast<const u32x4*>(unit + (wave + 4 * s) * (ZL::PIECES * 1024) + j * 1024 + lane * 16);
+
+  // this lane's 16 values of each of its sub-blocks, as d(logits) in the operand dtype
+  T dz[kSubPerWave][16];
+#pragma unroll
+  for (int s = 0; s < kSubPerWave; ++s) {
+    const int sb = wave + 4 * s;
+    const int R = (sb / ZL::VSUB) * 32 + t32;       // token row inside the unit
+    const int c0 = (sb % ZL::VSUB) * 32;            // first vocabulary entry of the sub-block inside the unit
+    const int t = rb * kBlockRows + R;
+    float glp = 0.f, gen = 0.f, lse = 0.f, ent = 0.f;
+    int lab = -1;
+    if (t < p.Tc) {
+      glp = p.g_lp[t];
+      gen = p.g_ent ? p.g_ent[t] : 0.f;
+      lse = p.lse[t];
+      ent = p.g_ent ? p.entropy[t] : 0.f;
+      const int64_t rel = p.labels[t] - p.label_offset - ((int64_t)ks * E + c0);   // relative to the sub-block
+      lab = (rel >= 0 && rel < 32) ? (int)rel : -1;
+    }
+    const bool live = glp != 0.f || gen != 0.f;     // rows past the chunk and rows without a gradient give zeros
+    const float lse2 = lse * kLog2e;
+#pragma unroll
+    for (int j = 0; j < ZL::PIECES; ++j) {
+      const ZT* in = reinterpret_cast<const ZT*>(&raw[s][j]);
+#pragma unroll
+      for (int e = 0; e < ZL::kPerPiece; ++e) {
+        const int c32 = ZL::col_of(h, j, e);
+        float d = 0.f;
+        if (live) {
+          const float zraw = (float)in[e];
           const float pr = __builtin_amdgcn_exp2f(fmaf(zraw, p.c, -lse2));
           const float logp = fmaf(zraw, it, -lse);
-          float d = -it * pr * fmaf(gen, logp + ent, glp);
-          if (v + j == lab) d += it * glp;
-          if (v + j >= p.V) d = 0.f;
-          vals[j] = (T)d;
+          d = -it * pr * fmaf(gen, logp + ent, glp);
+          if (c32 == lab) d += it * glp;
+          if (ks * E + c0 + c32 >= p.V) d = 0.f;    // vocabulary padding columns
         }
+        dz[s][j * ZL::kPerPiece + e] = (T)d;
       }
-      *reinterpret_cast<u32x4*>(z + blocked_index<T>(t, v, p.ldv / kE)) = *reinterpret_cast<const u32x4*>(vals);
     }
+  }
+
+  // pass 1: [token][vocab] through LDS, back over the unit as the K-blocked dz operand
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) tile[c * VEC + j][rr] = vals[j];
+  for (int s = 0; s < kSubPerWave; ++s) {
+    const int sb = wave + 4 * s;
+    const int R = (sb / ZL::VSUB) * 32 + t32;
+    const int c0 = (sb % ZL::VSUB) * 32;
+    // registers 4m .. 4m+3 are consecutive vocabulary entries: 4 * sizeof(T) bytes of the token's row
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int byte = (c0 + 8 * m + 4 * h) * (int)sizeof(T);
+      char* dst = tile + R * kRowBytes + (((byte >> 4) ^ (R & 7)) << 4) + (byte & 15);
+      if (sizeof(T) == 2) *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(&dz[s][4 * m]);
+      else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(&dz[s][4 * m]);
+    }
+  }
+  __syncthreads();     // also: every thread has its part of the unit in registers before anyone overwrites it
+  for (int pc = threadIdx.x; pc < kBlockRows * kChunksPerRow; pc += 256) {
+    const int R = pc >> 3, q = pc & 7;              // row R, 16-byte chunk q of the operand is piece R * 8 + q
+    *reinterpret_cast<u32x4*>(unit + pc * 16) = *reinterpret_cast<const u32x4*>(tile + R * kRowBytes + ((q ^ (R & 7)) << 4));
   }
   __syncthreads();
-  for (int rr = r; rr < 64; rr += RPP) {
-    const int v = v0 + rr;
-    const int t = t0 + c * VEC;
-    if (v < p.V && t < p.ldt)
-      *reinterpret_cast<u32x4*>(dzT + blocked_index<T>(v, t, p.ldt / kE)) = *reinterpret_cast<const u32x4*>(&tile[rr][c * VEC]);
+
+  // pass 2: [vocab][token] through LDS, out to the K-blocked dzT operand (vocabulary row v, token slabs of E)
+#pragma unroll
+  for (int s = 0; s < kSubPerWave; ++s) {
+    const int sb = wave + 4 * s;
+    const int R = (sb / ZL::VSUB) * 32 + t32;
+    const int c0 = (sb % ZL::VSUB) * 32;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      *reinterpret_cast<T*>(tile + (c0 + 8 * (r >> 2) + 4 * h + (r & 3)) * kTPitch + R * (int)sizeof(T)) = dz[s][r];
+  }
+  __syncthreads();
+  T* dzT = static_cast<T*>(p.dzT);
+  const int64_t n_tslab = p.ldt / E;
+  for (int pc = threadIdx.x; pc < E * (kBlockRows / VEC); pc += 256) {
+    const int sl = pc / (E * kChunksPerRow);        // token slab inside the unit
+    const int c = (pc / kChunksPerRow) % E;         // vocabulary row inside the unit
+    const int q = pc % kChunksPerRow;
+    const int v = ks * E + c;
+    const int tok = rb * kBlockRows + sl * E + q * VEC;
+    if (v < p.V && tok < p.ldt)
+      *reinterpret_cast<u32x4*>(dzT + blocked_index<T>(v, tok, n_tslab)) =
+          *reinterpret_cast<const u32x4*>(tile + c * kTPitch + (sl * E + q * VEC) * (int)sizeof(T));
   }
 }
 
@@ -236,7 +299,36 @@ template <typename OutT> __device__ __forceinline__ OutT cvt_out(float v);
 template <> __device__ __forceinline__ float cvt_out<float>(float v) { return v; }
 template <> __device__ __forceinline__ __bf16 cvt_out<__bf16>(float v) { return (__bf16)v; }
 
-// Output tile (mt, nt) from the accumulators: C (+)= acc, or the fp32 partial of K range `ks`.
+// Accumulators of output tile (m0, n0) before its K loop: zeros, or - when the GEMM adds to C and one
+// workgroup owns the whole K range of the tile - the tile's current contents.  Reading C here instead of
+// in the epilogue puts the loads' latency in front of the K loop, where the first operand slabs are in
+// flight anyway, and leaves the epilogue a pure store.
+template <typename T, typename OutT>
+__device__ __forceinline__ void gemm_init_tile(const GemmParams& p, f32x16 (&acc)[HeadTile<T>::MI][HeadTile<T>::NI],
+                                               int m0, int n0, int a_rows, int b_rows) {
+  using Tile = HeadTile<T>;
+  constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave % 2, wn = wave / 2;
+  const bool from_c = p.accumulate && p.k_split == 1;
+  const OutT* C = static_cast<const OutT*>(p.C);
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+    const int col = wn * WN + ni * 32 + (lane & 31);
+    const bool col_ok = from_c && col < b_rows;
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = wm * WM + mi * 32 + acc_row(r, lane);
+        acc[mi][ni][r] = (col_ok && row < a_rows) ? (float)C[(int64_t)(m0 + row) * p.ldc + (n0 + col)] : 0.f;
+      }
+  }
+}
+
+// Output tile (mt, nt) from the accumulators: C = acc (the accumulators already hold C's previous
+// contents when the GEMM adds to it, see gemm_init_tile), or the fp32 partial of K range `ks`.
 template <typename T, typename OutT>
 __device__ __forceinline__ void gemm_store_tile(const GemmParams& p, f32x16 (&acc)[HeadTile<T>::MI][HeadTile<T>::NI],
                                                 int m0, int n0, int a_rows, int b_rows, int ks) {
@@ -272,10 +364,7 @@ __device__ __forceinline__ void gemm_store_tile(const GemmParams& p, f32x16 (&ac
       for (int r = 0; r < 16; ++r) {
         const int row = wm * WM + mi * 32 + acc_row(r, lane);
         if (row < a_rows) {
-          OutT* dst = C + (int64_t)(m0 + row) * p.ldc + (n0 + col);
-          float v = acc[mi][ni][r];
-          if (p.accumulate) v += (float)*dst;
-          *dst = cvt_out<OutT>(v);
+          C[(int64_t)(m0 + row) * p.ldc + (n0 + col)] = cvt_out<OutT>(acc[mi][ni][r]);
         }
       }
   }
@@ -310,12 +399,7 @@ __global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
       const int m1 = m0 + 256;
       const int next_rows = (p.M - m1) < 256 ? (p.M - m1) : 256;
       const T* A = static_cast<const T*>(p.A) + (int64_t)mt * p.a_kslabs * kSlabElems;
-#pragma unroll
-      for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+      gemm_init_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows);
       Tile::run(acc, Tile::Operand::blocked(A, a_rows), Tile::Operand::blocked(B, b_rows), p.K, lds, st,
                 (mt + 1 < mt_end) ? A + p.a_kslabs * kSlabElems : nullptr, next_rows, true);
       gemm_store_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows, 0);
@@ -333,12 +417,7 @@ __global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
   const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
   const int k0 = ks * p.k_per_split;
   const int k_len = (p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split;
-#pragma unroll
-  for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+  gemm_init_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows);
 
   constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;
   const int64_t s0 = k0 / Tile::kSlabK;   // first slab of this K range
@@ -530,7 +609,7 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream, int64_t 
       q.ldv = (int)ldz;
       q.c = a->inv_temperature * kLog2e;
       q.inv_temperature = a->inv_temperature;
-      dim3 grid((unsigned)((ldt + 63) / 64), (unsigned)((pl.ldv + 63) / 64));
+      dim3 grid((unsigned)((tc + kBlockRows - 1) / kBlockRows), (unsigned)(ldz / Elem<T>::kSlabK));
       hipLaunchKernelGGL(dz_from_z_kernel<T>, grid, dim3(256), 0, stream, q);
       rc = check_launch("dz_from_z_kernel");
       if (rc) return rc;

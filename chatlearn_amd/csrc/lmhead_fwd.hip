@@ -6,8 +6,10 @@
 // target logit) for its own tokens across all vocabulary tiles of its split.
 // A workgroup owns one block of 256 tokens and one contiguous range of
 // vocabulary tiles ("split"); a second small kernel merges the splits with an
-// exact rescale and writes logprob / entropy / rowmax / lse.  Logits never go
-// to memory.
+// exact rescale and writes logprob / entropy / rowmax / lse.  Logits go to
+// memory only when the caller asks for a chunk's raw logits to be kept for the
+// backward; they then leave straight from the accumulators, 16 bytes per lane,
+// in the accumulators' own order (see ZNative).
 //
 // Algorithmic work: 2*T*H*V flop; bytes 2*T*H + 2*V*H (bf16) + 16*T.
 #include "common.hpp"
@@ -16,7 +18,6 @@
 namespace clgrpo {
 
 constexpr int kFwdBM = 256, kFwdBN = 256;
-constexpr int kZRow = kFwdBM * 2 + 16;   // bytes per token row of a 16-bit logits tile turned through LDS (padded)
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct FwdParams {
@@ -27,27 +28,26 @@ struct FwdParams {
   int T, H, V;
   int n_tb, n_split, tiles_per_split, n_vt;
   float c;  // inv_temperature * log2(e)
-  void* z_out;   // optional raw logits in the input dtype, K-blocked: rows x ldz, see blocked_index
+  void* z_out;   // optional raw logits, z-native layout (see ZNative): rows x ldz entries of KeptLogit<T>
   int64_t ldz;
   const int32_t* z_row_map;  // optional [T]: destination row per token, < 0: not stored
   int z_rows;                // rows of z_out; mapped rows outside [0, z_rows) are not stored
   float4* part;  // [n_split][T]: (max raw, sum 2^{(z-max) c}, sum 2^{(z-max) c} z raw, target raw)
 };
 
-template <typename T> struct Pack4;
-template <> struct Pack4<float> {
-  typedef float4 type;
-  __device__ static __forceinline__ type make(float a, float b, float c, float d) { return make_float4(a, b, c, d); }
-};
-template <> struct Pack4<__bf16> {
-  typedef uint2 type;
-  __device__ static __forceinline__ type make(float a, float b, float c, float d) {
-    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-    bf16x2 lo = {(__bf16)a, (__bf16)b};
-    bf16x2 hi = {(__bf16)c, (__bf16)d};
-    return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
-  }
-};
+// 16 bytes of kept logits from consecutive accumulator registers.
+template <typename ZT> __device__ __forceinline__ u32x4 pack_piece(const f32x16& a, int first);
+template <> __device__ __forceinline__ u32x4 pack_piece<float>(const f32x16& a, int first) {
+  f32x4 v = {a[first], a[first + 1], a[first + 2], a[first + 3]};
+  return __builtin_bit_cast(u32x4, v);
+}
+template <> __device__ __forceinline__ u32x4 pack_piece<_Float16>(const f32x16& a, int first) {
+  typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+  f16x8 v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (_Float16)a[first + e];     // round to nearest even
+  return __builtin_bit_cast(u32x4, v);
+}
 
 __device__ __forceinline__ void merge_state(float& m, float& s, float& u, float om, float os,
                                             float ou, float c) {
@@ -111,19 +111,20 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
-    // The K loop requests the first slabs of the next vocabulary tile during its last two slab
-    // periods, except where 16-bit logits are turned through LDS after it.
-    constexpr bool kZViaLds = STORE_Z && sizeof(T) == 2;
+    // The K loop requests the first slabs of the next vocabulary tile during its last two slab periods.
     const bool has_next = vt + 1 < vt_end;
     const int v1 = v0 + kFwdBM;
     const int next_rows = (p.V - v1) < kFwdBM ? (p.V - v1) : kFwdBM;
     const T* next_w = weight + (int64_t)v1 * p.H;
     Tile::run(acc, Tile::Operand::row_major(weight + (int64_t)v0 * p.H, p.H, a_rows),
-              Tile::Operand::row_major(hidden, p.H, b_rows), p.H, lds, st,
-              (has_next && !kZViaLds) ? next_w : nullptr, next_rows, true);
+              Tile::Operand::row_major(hidden, p.H, b_rows), p.H, lds, st, has_next ? next_w : nullptr, next_rows, true);
 
     if (STORE_Z) {
-      // Raw logits for the backward; the padding columns past V are stored as zeros.
+      // Raw logits for the backward, straight from the accumulators: per 32x32 block a lane stores its
+      // 16 values as 16-byte pieces, each piece of the 64 lanes one contiguous KB (z-native layout).
+      // The padding columns past V are stored as zeros.
+      typedef typename KeptLogit<T>::type ZT;
+      typedef ZNative<ZT> ZL;
       if (a_rows < kFwdBM) {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
@@ -133,52 +134,19 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
             for (int r = 0; r < 16; ++r)
               if (wm * WM + mi * 32 + acc_row(r, lane) >= a_rows) acc[mi][ni][r] = 0.f;
       }
-      T* z = static_cast<T*>(p.z_out);
-      typedef typename Pack4<T>::type P4;
-      if (kZViaLds) {
-        // 16-bit logits: turn the tile through LDS (free between two K loops) so that every token
-        // row leaves as whole 16-byte pieces of one contiguous 512-byte run.
+      char* z = static_cast<char*>(p.z_out);
+      const int64_t n_kslab = p.ldz / ZL::kSlabElems;
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni) {
-          char* row = lds + (wn * WN + ni * 32 + (lane & 31)) * kZRow;
+      for (int ni = 0; ni < NI; ++ni) {
+        if (zrow[ni] < 0) continue;
 #pragma unroll
-          for (int mi = 0; mi < MI; ++mi)
+        for (int mi = 0; mi < MI; ++mi) {
+          const int v_blk = v0 + wm * WM + mi * 32;
+          if (v_blk >= p.ldz) continue;
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-              *reinterpret_cast<P4*>(row + (wm * WM + mi * 32 + 8 * q + 4 * (lane >> 5)) * 2) =
-                  Pack4<T>::make(acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
-                                 acc[mi][ni][4 * q + 3]);
-        }
-        __syncthreads();
-        const int chunk = threadIdx.x & 31;          // 16-byte piece within the 512-byte row
-        const int v_idx = v0 + chunk * 8;
-        if (v_idx < p.ldz) {
-          const int64_t n_kslab = p.ldz / Tile::kSlabK;
-          for (int r = threadIdx.x >> 5; r < kFwdBN; r += Tile::kThreads / 32) {
-            const int tok = t0 + r;
-            int dst = (tok < p.T) ? (p.z_row_map ? p.z_row_map[tok] : tok) : -1;
-            if (dst >= p.z_rows) dst = -1;
-            if (dst >= 0)
-              *reinterpret_cast<u32x4*>(z + blocked_index<T>(dst, v_idx, n_kslab)) =
-                  *reinterpret_cast<const u32x4*>(lds + r * kZRow + chunk * 16);
-          }
-        }
-        __syncthreads();   // the next K loop refills the same LDS
-      } else {
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni) {
-          if (zrow[ni] >= 0) {
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-              for (int q = 0; q < 4; ++q) {
-                const int v_idx = v0 + wm * WM + mi * 32 + 8 * q + 4 * (lane >> 5);
-                if (v_idx < p.ldz)
-                  *reinterpret_cast<P4*>(z + blocked_index<T>(zrow[ni], v_idx, p.ldz / Tile::kSlabK)) =
-                      Pack4<T>::make(acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
-                                     acc[mi][ni][4 * q + 3]);
-              }
-          }
+          for (int j = 0; j < ZL::PIECES; ++j)
+            *reinterpret_cast<u32x4*>(z + ZL::piece_offset(zrow[ni], v_blk >> 5, n_kslab, lane >> 5, j)) =
+                pack_piece<ZT>(acc[mi][ni], j * ZL::kPerPiece);
         }
       }
     }
@@ -364,9 +332,7 @@ static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream, int64
   p.ldz = a->ld_saved;
   p.z_row_map = a->saved_row_map;
   p.z_rows = (int)a->saved_rows;
-  // the K loop's two stages, or the logits tile when it is turned through LDS
-  constexpr int kZTile = (STORE_Z && sizeof(T) == 2) ? kFwdBN * kZRow : 0;
-  constexpr int lds_bytes = Tile::kLdsBytes > kZTile ? Tile::kLdsBytes : kZTile;
+  constexpr int lds_bytes = Tile::kLdsBytes;
   int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&lmhead_fwd_kernel<T, STORE_Z>), lds_bytes, "lmhead_fwd_kernel");
   if (rc) return rc;
   int grid = p.n_tb * p.n_split;

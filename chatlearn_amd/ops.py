@@ -50,9 +50,11 @@ def _round_up(x: int, m: int) -> int:
 
 
 def saved_logits_buffer(T: int, V: int, dtype, device) -> torch.Tensor:
-    """An (uninitialised) buffer the forward can store raw logits in for the backward: T rows rounded
-    up to whole blocks of 256 by the padded vocabulary extent.  Its layout is the library's K-blocked
-    one (``saved_logits_rowmajor`` turns it back into rows)."""
+    """An (uninitialised) buffer the forward can keep raw logits in for the backward: T rows rounded
+    up to whole blocks of 256 by the padded vocabulary extent, elements of the size of ``dtype``.  Its
+    contents are opaque (``saved_logits_rowmajor`` decodes them): the forward stores the logits in the
+    order of its accumulators, 16-bit inputs as IEEE half; the backward overwrites the buffer with
+    d(logits) in the layout of its GEMM operands."""
     return torch.empty(_round_up(max(T, 1), 256), _lib.lib().clgrpo_saved_logits_ld(V), dtype=dtype, device=device)
 
 
@@ -65,8 +67,21 @@ def _unblock(buf: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
 
 
 def saved_logits_rowmajor(buf: torch.Tensor, rows: int, V: int) -> torch.Tensor:
-    """The first ``rows`` kept rows as an ordinary [rows, V] tensor (a copy; for inspection and tests)."""
-    return _unblock(buf, rows, V)
+    """The first ``rows`` kept rows as an ordinary fp32 [rows, V] tensor (a copy; for inspection and tests).
+    Decodes the forward's layout: 32 KB units of 256 rows x one 128-byte slab of vocabulary; inside a unit
+    sub-blocks of 32 rows x 32 entries, each stored as [16-byte piece][lane half][row][values] where value
+    r of lane half h is vocabulary entry 8 * (r // 4) + 4 * h + r % 4 of the sub-block."""
+    es = buf.element_size()
+    z = buf.view(torch.float16) if es == 2 else buf
+    e = 128 // es                       # vocabulary entries per unit
+    vsub, pieces = e // 32, es          # sub-blocks along the vocabulary, 16-byte pieces per lane
+    per = 16 // pieces                  # values per piece
+    nb, ld = buf.shape[0] // 256, buf.shape[1]
+    z = z.reshape(nb, ld // e, 8, vsub, pieces, 2, 32, per)           # unit: [rs][vs][piece j][h][t32][value]
+    z = z.permute(0, 2, 6, 1, 3, 4, 7, 5)                             # [nb][rs][t32][ks][vs][j][value][h]
+    z = z.reshape(nb, 8, 32, ld // e, vsub, pieces * per // 4, 4, 2)  # register r = 4 * q + i -> [q][i][h]
+    z = z.permute(0, 1, 2, 3, 4, 5, 7, 6)                             # entry = 8 * q + 4 * h + i
+    return z.reshape(nb * 256, ld)[:rows, :V].float()
 
 
 def weight_t_buffer(weight: torch.Tensor) -> torch.Tensor:

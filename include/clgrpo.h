@@ -58,14 +58,17 @@ typedef struct {
   float* lse;              /* [T] out, fp32 (logsumexp_v z); required */
   void* workspace;
   size_t workspace_bytes;
-  void* saved_logits;      /* optional out, `dtype`: the raw logits hidden.W^T (before the temperature), for a
-                              later clgrpo_lmhead_bwd of the SAME rows that then skips the recomputation.
-                              NULL: nothing is stored.  Callers bound its size by processing a micro-batch in
-                              token chunks.  The buffer is opaque to the caller: ceil(rows / 256) * 256 rows of
-                              ld_saved elements, laid out in blocks of 256 rows; inside a block the 128-byte K
-                              slabs of all 256 rows follow one another, so element (row, k) lives at
+  void* saved_logits;      /* optional out: the raw logits hidden.W^T (before the temperature), for a later
+                              clgrpo_lmhead_bwd of the SAME rows that then skips the recomputation.  NULL: nothing
+                              is stored.  Callers bound its size by processing a micro-batch in token chunks.
+                              The buffer is opaque to the caller: ceil(rows / 256) * 256 rows of ld_saved elements
+                              of sizeof(dtype) bytes.  The forward fills it in the order of its accumulators
+                              (32 KB units of 256 rows x 128 bytes of vocabulary, inside a unit 32 x 32 sub-blocks
+                              stored as 16-byte pieces per lane; 16-bit inputs keep their logits as IEEE half);
+                              the backward overwrites every unit in place with d(logits) as the K-blocked operand
+                              of its GEMMs: element (row, k) at
                               (((row / 256) * (ld_saved / E) + k / E) * 256 + row % 256) * E + k % E,
-                              E = 128 / sizeof(dtype).  This is the operand layout of the backward GEMMs. */
+                              E = 128 / sizeof(dtype). */
   int64_t ld_saved;        /* K extent in elements, a multiple of 64, >= clgrpo_saved_logits_ld(V) */
   const int32_t* saved_row_map; /* optional [T]: row of saved_logits that receives token t's logits, or a
                               negative value to store nothing for t (tokens whose upstream gradient is
@@ -104,9 +107,9 @@ typedef struct {
   int32_t accumulate_dweight; /* nonzero: dweight += ; zero: dweight = */
   void* workspace;
   size_t workspace_bytes;   /* sets the token chunk: see clgrpo_lmhead_bwd_workspace_bytes */
-  void* saved_logits;       /* optional in/out: logits stored by clgrpo_lmhead_fwd for these rows (same opaque
-                               blocked layout, ceil(T / 256) * 256 rows of ld_saved elements).  Overwritten in
-                               place with d(logits); the recomputation is skipped. */
+  void* saved_logits;       /* optional in/out: logits stored by clgrpo_lmhead_fwd for these rows (the same opaque
+                               buffer, ceil(T / 256) * 256 rows of ld_saved elements).  Overwritten in place
+                               with d(logits); the recomputation is skipped. */
   int64_t ld_saved;
   void* weight_t;           /* optional, `dtype`: caller-kept W^T in the same blocked layout (ceil(H / 256) * 256
                                rows of clgrpo_saved_logits_ld(V) elements), so that several calls with the same

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 CFG = synthetic.CONFIGS["c2"]
 # Smallest fraction of bf16 dW entries that must sit inside |err| <= atol + 1e-2 |ref|, atol = 1e-2
 # median|ref| (see tests/test_gpu_head_step.py::DW_FRAC_BF16 for why it is not 1).
-DW_FRAC_BF16 = 0.94
+DW_FRAC_BF16 = 0.999
 
 
 @pytest.fixture(scope="module")
@@ -258,7 +258,7 @@ def test_full_head_shapes_forward_backward_against_the_float64_oracle(dev, name,
     assert_close_rel(dh, rdh, 1e-2, f"{name} dhidden")
     assert_close_rel(dw, rdw, 1e-2, f"{name} dweight")
     assert_rows_rel_l2(dh, rdh, 1e-2, f"{name} dhidden rows")
-    assert_rows_rel_l2(dw, rdw, 2e-2, f"{name} dweight rows")
+    assert_rows_rel_l2(dw, rdw, 1e-2, f"{name} dweight rows")
     ours_dh = assert_contract(dh, rdh, 1e-2, f"{name} dhidden")
     ours_dw = assert_contract(dw, rdw, 1e-2, f"{name} dweight", min_frac=DW_FRAC_BF16)
     if name == "c2":

@@ -39,7 +39,7 @@ CASES = [
 # 1e-2 median|ref|).  The rest are entries whose terms cancel to well below the tensor's typical
 # magnitude; their error is the bf16 rounding of d(logits) (2^-9 relative per term, the same rounding the
 # reference's bf16 autograd applies), not a wrong term: the row-wise L2 and max-norm bounds above hold at 1e-2.
-DW_FRAC_BF16 = 0.99
+DW_FRAC_BF16 = 0.995
 # fp32: the same cancelling entries against fp32 accumulation order, a few in 10^4.
 DW_FRAC_FP32 = 0.999
 
@@ -123,7 +123,7 @@ def test_kept_logits_backward_equals_recompute(dev):
     lp2, ent2, _, lse2 = ops.lmhead_forward(hidden, weight, labels, 0.8)
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2)            # storing logits does not change the statistics
     z = torch.nn.functional.linear(hidden.float(), weight.float())
-    assert_close_rel(ops.saved_logits_rowmajor(zbuf, T, V), z, 2 ** -8, "stored logits")   # bf16 rounding of the raw logits
+    assert_close_rel(ops.saved_logits_rowmajor(zbuf, T, V), z, 2 ** -11, "stored logits")   # kept as IEEE half: 2^-11 relative
     assert (ops.saved_logits_rowmajor(zbuf, T, zbuf.shape[1])[:, V:] == 0).all()         # vocabulary padding columns
     dh1, dw1 = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_en, 0.8)
     dh2, dw2 = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_en, 0.8, saved_logits=zbuf)
