@@ -222,25 +222,31 @@ struct GemmTile {
   // outstanding ones explicitly (s_waitcnt vmcnt(0), the other counters left alone).
   __device__ static __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-  // acc[mi][ni] must be zeroed by the caller.  `a` / `b` describe the tile's rows from K offset 0;
-  // K must be a multiple of kSlabK and every row 16-byte aligned.  With a_next != nullptr the last
-  // two slab periods request the first two slabs of the next K loop (A rows from a_next with
-  // a_next_rows valid rows, same layout as `a`; same B), and LDS stays in use on return; otherwise,
-  // with release_lds, all loads have landed and every wave is past its last fragment read on return.
+  // acc[mi][ni] must be initialised by the caller.  `a` / `b` describe the tile's rows from K offset 0;
+  // K must be a multiple of kSlabK and every row 16-byte aligned.  With next != nullptr the last
+  // two slab periods request the first two slabs of the next K loop, which keeps one operand and
+  // takes the other's rows from `next` (next_rows valid rows, same layout as the operand it replaces:
+  // A unless next_is_b), and LDS stays in use on return; otherwise, with release_lds, all loads have
+  // landed and every wave is past its last fragment read on return.
   __device__ static __forceinline__ void run(f32x16 (&acc)[MI][NI], const Operand& a, const Operand& b, int K,
-                                             char* lds, Stream& st, const T* a_next, int a_next_rows,
-                                             bool release_lds) {
+                                             char* lds, Stream& st, const T* next, int next_rows,
+                                             bool release_lds, bool next_is_b = false) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int wm = wave % WAVES_M;
     const int wn = wave / WAVES_M;
     const Loader L = make_loader(a, b);
     const int nslab = K / kSlabK;
-    const bool stream_on = a_next != nullptr && nslab >= 2;
+    const bool stream_on = next != nullptr && nslab >= 2;
     Loader LN = L;
     if (stream_on) {
-      LN.a_ptr = reinterpret_cast<const char*>(a_next);
-      LN.a_bytes = a_next_rows * a.row_bytes;
+      if (next_is_b) {
+        LN.b_ptr = reinterpret_cast<const char*>(next);
+        LN.b_bytes = next_rows * b.row_bytes;
+      } else {
+        LN.a_ptr = reinterpret_cast<const char*>(next);
+        LN.a_bytes = next_rows * a.row_bytes;
+      }
     }
 
     const int fr_swz = (lane & 7) ^ ((lane >> 3) & 1);

@@ -280,7 +280,16 @@ __global__ __launch_bounds__(256) void dz_from_z_kernel(DzFromZParams p) {
   }
 }
 
-// C[m][n] (+)= sum_k A[m][k] B[n][k];  C row-major with leading dimension ldc, A and B K-blocked.
+// C (+)= A B^T with A [M x K] and B [N x K] K-blocked, C row-major in one of two orientations:
+//   kMContig = false: C[m][n], ld = ldc.  The N index runs along the lanes of an accumulator block
+//     (see gemm_core.hpp), so one store instruction writes whole 128-byte lines (32 lanes x 4 bytes,
+//     two rows): the orientation for fp32 outputs (dW: A = dz^T, B = hidden^T).
+//   kMContig = true:  C[n][m], ld = ldc.  The M index runs along a lane's registers, so a lane owns 4
+//     consecutive elements of a row per register quad: one 8-byte access instead of four 2-byte ones
+//     for 16-bit outputs (dhidden: A = W^T, B = dz).
+// Measured on the Qwen3-8B head: fp32 out, C[n][m] with 16-byte accesses (32 rows x 32 bytes per
+// instruction) is 4 % slower than C[m][n] with 4-byte ones (2 rows x 128 bytes): whole lines matter
+// more than the number of memory instructions; bf16 out gains 2 % from the 8-byte accesses.
 struct GemmParams {
   const void* A;      // M x K, K-blocked with a_kslabs slabs per row block
   const void* B;      // N x K, K-blocked with b_kslabs slabs per row block
@@ -291,118 +300,189 @@ struct GemmParams {
   int accumulate;
   int k_split;        // > 1: work item = (tile, K range); fp32 partial tiles go to `partial`
   int k_per_split;    // K extent of one range, a multiple of the slab
-  int n_walk;         // > 0: workgroups walk runs of m tiles (see gemm_nt_kernel); needs k_split == 1
-  float* partial;     // [k_split][M][N] fp32, row stride N
+  int n_walk;         // > 0: workgroups walk runs of tiles (see gemm_nt_kernel); needs k_split == 1
+  float* partial;     // [k_split] copies of C's shape in fp32, densely packed (row stride N or M)
 };
 
-template <typename OutT> __device__ __forceinline__ OutT cvt_out(float v);
-template <> __device__ __forceinline__ float cvt_out<float>(float v) { return v; }
-template <> __device__ __forceinline__ __bf16 cvt_out<__bf16>(float v) { return (__bf16)v; }
+// Addresses of a 256 x 256 output tile for the accumulator layout: a range-checked buffer descriptor over
+// the tile's valid rows, one per-lane byte offset per 32-wide block of the lane dimension, and an offset
+// per accumulator register (kMContig: per register quad, a compile-time constant; otherwise a uniform
+// multiple of the row pitch).  Elements outside the tile fall outside the descriptor or are skipped as a
+// whole quad (M extents are multiples of 64 here): loads of them give 0 and stores are dropped, so no
+// per-element branch or 64-bit address is needed.
+template <typename T, typename OutT, bool kMContig>
+struct TileAddr {
+  using Tile = HeadTile<T>;
+  static constexpr int ES = (int)sizeof(OutT);
+  __amdgpu_buffer_rsrc_t rsrc;
+  int voff[Tile::NI];
+  int row_bytes, m_first, a_rows;
+  __device__ __forceinline__ TileAddr(OutT* base, int64_t ld, int m0, int n0, int a_rows_, int b_rows) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave % 2, wn = wave / 2;
+    row_bytes = (int)(ld * (int64_t)ES);
+    m_first = wm * Tile::WM;
+    a_rows = a_rows_;
+    const int rows = kMContig ? b_rows : a_rows_, cols = kMContig ? a_rows_ : b_rows;
+    const int bytes = rows > 0 ? (rows - 1) * row_bytes + cols * ES : 0;
+    OutT* origin = kMContig ? base + (int64_t)n0 * ld + m0 : base + (int64_t)m0 * ld + n0;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(origin), 0, bytes, 0x00020000);
+#pragma unroll
+    for (int ni = 0; ni < Tile::NI; ++ni) {
+      const int n = wn * Tile::WN + ni * 32 + (lane & 31);
+      const int m = m_first + 4 * (lane >> 5);
+      voff[ni] = n < b_rows ? (kMContig ? n * row_bytes + m * ES : m * row_bytes + n * ES) : 0x7f000000;
+    }
+  }
+  // offset of register r of block row mi from voff (rows 8 * (r / 4) + r % 4 of the block, plus the lane half's 4)
+  __device__ __forceinline__ int reg_off(int mi, int r) const {
+    const int dm = mi * 32 + 8 * (r >> 2) + (r & 3);
+    return kMContig ? dm * ES : dm * row_bytes;
+  }
+  __device__ __forceinline__ bool quad_ok(int mi, int q) const { return m_first + mi * 32 + 8 * q < a_rows; }
+};
+
+__device__ __forceinline__ float elem_load(const __amdgpu_buffer_rsrc_t& rsrc, int voff, int soff, float*) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, soff, 0));
+}
+__device__ __forceinline__ float elem_load(const __amdgpu_buffer_rsrc_t& rsrc, int voff, int soff, __bf16*) {
+  return (float)__builtin_bit_cast(__bf16, __builtin_amdgcn_raw_buffer_load_b16(rsrc, voff, soff, 0));
+}
+__device__ __forceinline__ void elem_store(float v, const __amdgpu_buffer_rsrc_t& rsrc, int voff, int soff, float*) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), rsrc, voff, soff, 0);
+}
+__device__ __forceinline__ void elem_store(float v, const __amdgpu_buffer_rsrc_t& rsrc, int voff, int soff, __bf16*) {
+  __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, (__bf16)v), rsrc, voff, soff, 0);
+}
+__device__ __forceinline__ void quad_load(f32x16& a, int q, const __amdgpu_buffer_rsrc_t& rsrc, int voff, float*) {
+  const f32x4 v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 0, 0));
+  a[4 * q] = v[0]; a[4 * q + 1] = v[1]; a[4 * q + 2] = v[2]; a[4 * q + 3] = v[3];
+}
+__device__ __forceinline__ void quad_load(f32x16& a, int q, const __amdgpu_buffer_rsrc_t& rsrc, int voff, __bf16*) {
+  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+  const bf16x4 v = __builtin_bit_cast(bf16x4, __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, 0, 0));
+  a[4 * q] = (float)v[0]; a[4 * q + 1] = (float)v[1]; a[4 * q + 2] = (float)v[2]; a[4 * q + 3] = (float)v[3];
+}
+__device__ __forceinline__ void quad_store(const f32x16& a, int q, const __amdgpu_buffer_rsrc_t& rsrc, int voff, float*) {
+  const f32x4 v = {a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, voff, 0, 0);
+}
+__device__ __forceinline__ void quad_store(const f32x16& a, int q, const __amdgpu_buffer_rsrc_t& rsrc, int voff, __bf16*) {
+  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+  typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+  const bf16x4 v = {(__bf16)a[4 * q], (__bf16)a[4 * q + 1], (__bf16)a[4 * q + 2], (__bf16)a[4 * q + 3]};
+  __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), rsrc, voff, 0, 0);
+}
+
+template <typename T, typename OutT, bool kMContig, typename AccT>
+__device__ __forceinline__ void tile_load(const TileAddr<T, OutT, kMContig>& at, AccT& acc) {
+  using Tile = HeadTile<T>;
+#pragma unroll
+  for (int ni = 0; ni < Tile::NI; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < Tile::MI; ++mi)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (!at.quad_ok(mi, q)) continue;
+        if (kMContig) quad_load(acc[mi][ni], q, at.rsrc, at.voff[ni] + at.reg_off(mi, 4 * q), (OutT*)nullptr);
+        else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[mi][ni][4 * q + i] = elem_load(at.rsrc, at.voff[ni], at.reg_off(mi, 4 * q + i), (OutT*)nullptr);
+        }
+      }
+}
+
+template <typename T, typename OutT, bool kMContig, typename AccT>
+__device__ __forceinline__ void tile_store(const TileAddr<T, OutT, kMContig>& at, const AccT& acc) {
+  using Tile = HeadTile<T>;
+#pragma unroll
+  for (int ni = 0; ni < Tile::NI; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < Tile::MI; ++mi)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (!at.quad_ok(mi, q)) continue;
+        if (kMContig) quad_store(acc[mi][ni], q, at.rsrc, at.voff[ni] + at.reg_off(mi, 4 * q), (OutT*)nullptr);
+        else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            elem_store(acc[mi][ni][4 * q + i], at.rsrc, at.voff[ni], at.reg_off(mi, 4 * q + i), (OutT*)nullptr);
+        }
+      }
+}
 
 // Accumulators of output tile (m0, n0) before its K loop: zeros, or - when the GEMM adds to C and one
 // workgroup owns the whole K range of the tile - the tile's current contents.  Reading C here instead of
 // in the epilogue puts the loads' latency in front of the K loop, where the first operand slabs are in
 // flight anyway, and leaves the epilogue a pure store.
-template <typename T, typename OutT>
+template <typename T, typename OutT, bool kMContig>
 __device__ __forceinline__ void gemm_init_tile(const GemmParams& p, f32x16 (&acc)[HeadTile<T>::MI][HeadTile<T>::NI],
                                                int m0, int n0, int a_rows, int b_rows) {
   using Tile = HeadTile<T>;
-  constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int wm = wave % 2, wn = wave / 2;
-  const bool from_c = p.accumulate && p.k_split == 1;
-  const OutT* C = static_cast<const OutT*>(p.C);
 #pragma unroll
-  for (int ni = 0; ni < NI; ++ni) {
-    const int col = wn * WN + ni * 32 + (lane & 31);
-    const bool col_ok = from_c && col < b_rows;
+  for (int mi = 0; mi < Tile::MI; ++mi)
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
+    for (int ni = 0; ni < Tile::NI; ++ni)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = wm * WM + mi * 32 + acc_row(r, lane);
-        acc[mi][ni][r] = (col_ok && row < a_rows) ? (float)C[(int64_t)(m0 + row) * p.ldc + (n0 + col)] : 0.f;
-      }
+      for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+  if (p.accumulate && p.k_split == 1) {
+    const TileAddr<T, OutT, kMContig> at(static_cast<OutT*>(p.C), p.ldc, m0, n0, a_rows, b_rows);
+    tile_load(at, acc);
   }
 }
 
-// Output tile (mt, nt) from the accumulators: C = acc (the accumulators already hold C's previous
-// contents when the GEMM adds to it, see gemm_init_tile), or the fp32 partial of K range `ks`.
-template <typename T, typename OutT>
+// Output tile from the accumulators: C = acc (the accumulators already hold C's previous contents
+// when the GEMM adds to it, see gemm_init_tile), or the fp32 partial of K range `ks`.
+template <typename T, typename OutT, bool kMContig>
 __device__ __forceinline__ void gemm_store_tile(const GemmParams& p, f32x16 (&acc)[HeadTile<T>::MI][HeadTile<T>::NI],
                                                 int m0, int n0, int a_rows, int b_rows, int ks) {
-  using Tile = HeadTile<T>;
-  constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int wm = wave % 2, wn = wave / 2;
   if (p.k_split > 1) {
-    float* P = p.partial + (int64_t)ks * p.M * p.N;
-#pragma unroll
-    for (int ni = 0; ni < NI; ++ni) {
-      const int col = wn * WN + ni * 32 + (lane & 31);
-      if (col >= b_rows) continue;
-#pragma unroll
-      for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = wm * WM + mi * 32 + acc_row(r, lane);
-          if (row < a_rows) P[(int64_t)(m0 + row) * p.N + (n0 + col)] = acc[mi][ni][r];
-        }
-    }
+    const TileAddr<T, float, kMContig> at(p.partial + (int64_t)ks * p.M * p.N, kMContig ? p.M : p.N, m0, n0, a_rows, b_rows);
+    tile_store(at, acc);
     return;
   }
-  OutT* C = static_cast<OutT*>(p.C);
-#pragma unroll
-  for (int ni = 0; ni < NI; ++ni) {
-    const int col = wn * WN + ni * 32 + (lane & 31);
-    if (col >= b_rows) continue;
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = wm * WM + mi * 32 + acc_row(r, lane);
-        if (row < a_rows) {
-          C[(int64_t)(m0 + row) * p.ldc + (n0 + col)] = cvt_out<OutT>(acc[mi][ni][r]);
-        }
-      }
-  }
+  const TileAddr<T, OutT, kMContig> at(static_cast<OutT*>(p.C), p.ldc, m0, n0, a_rows, b_rows);
+  tile_store(at, acc);
 }
 
-// Work item = (walk, n tile) when n_walk > 0: the workgroup walks a contiguous run of m tiles
-// for one n tile, so B rows stay the same and the K loops stream into each other (the next
-// tile's first slabs are requested while the current tile finishes and is stored).  Otherwise
-// work item = (K range, m tile, n tile), one K loop per workgroup.
-template <typename T, typename OutT>
+// Work item = (walk, fixed tile) when n_walk > 0: the workgroup keeps one operand's tile (A's m tile
+// when C is [n][m], B's n tile when C is [m][n]) and walks a contiguous run of tiles of the other, so the
+// K loops stream into each other (the next tile's first slabs are requested while the current tile
+// finishes and is stored).  Otherwise work item = (K range, m tile, n tile), one K loop per workgroup.
+template <typename T, typename OutT, bool kMContig>
 __global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
   using Tile = HeadTile<T>;
   constexpr int MI = Tile::MI, NI = Tile::NI;
+  constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;   // elements of one block's slab
   extern __shared__ __align__(16) char lds[];
 
   int item = xcd_remap(blockIdx.x, gridDim.x);
   f32x16 acc[MI][NI];
   if (p.n_walk > 0) {
-    if (item >= p.n_walk * p.n_nt) return;
-    int walk, nt;
-    grouped_tile(item, p.n_walk, p.n_nt, 4, walk, nt);
-    const int mt_begin = (int)((int64_t)walk * p.n_mt / p.n_walk);
-    const int mt_end = (int)((int64_t)(walk + 1) * p.n_mt / p.n_walk);
-    const int n0 = nt * 256;
-    const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
-    constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;   // elements of one block's slab
-    const T* B = static_cast<const T*>(p.B) + (int64_t)nt * p.b_kslabs * kSlabElems;
+    const int n_fixed = kMContig ? p.n_mt : p.n_nt;       // tiles of the operand that stays
+    const int n_moving = kMContig ? p.n_nt : p.n_mt;      // tiles of the operand that is walked
+    if (item >= p.n_walk * n_fixed) return;
+    int walk, ft;
+    grouped_tile(item, p.n_walk, n_fixed, 4, walk, ft);
+    const int w_begin = (int)((int64_t)walk * n_moving / p.n_walk);
+    const int w_end = (int)((int64_t)(walk + 1) * n_moving / p.n_walk);
     typename Tile::Stream st;
-    for (int mt = mt_begin; mt < mt_end; ++mt) {
-      const int m0 = mt * 256;
+    for (int wt = w_begin; wt < w_end; ++wt) {
+      const int mt = kMContig ? ft : wt, nt = kMContig ? wt : ft;
+      const int m0 = mt * 256, n0 = nt * 256;
       const int a_rows = (p.M - m0) < 256 ? (p.M - m0) : 256;
-      const int m1 = m0 + 256;
-      const int next_rows = (p.M - m1) < 256 ? (p.M - m1) : 256;
+      const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
+      const int moving_left = (kMContig ? p.N : p.M) - (wt + 1) * 256;
+      const int next_rows = moving_left < 256 ? moving_left : 256;
       const T* A = static_cast<const T*>(p.A) + (int64_t)mt * p.a_kslabs * kSlabElems;
-      gemm_init_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows);
+      const T* B = static_cast<const T*>(p.B) + (int64_t)nt * p.b_kslabs * kSlabElems;
+      const T* next = kMContig ? B + p.b_kslabs * kSlabElems : A + p.a_kslabs * kSlabElems;
+      gemm_init_tile<T, OutT, kMContig>(p, acc, m0, n0, a_rows, b_rows);
       Tile::run(acc, Tile::Operand::blocked(A, a_rows), Tile::Operand::blocked(B, b_rows), p.K, lds, st,
-                (mt + 1 < mt_end) ? A + p.a_kslabs * kSlabElems : nullptr, next_rows, true);
-      gemm_store_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows, 0);
+                (wt + 1 < w_end) ? next : nullptr, next_rows, true, /*next_is_b=*/kMContig);
+      gemm_store_tile<T, OutT, kMContig>(p, acc, m0, n0, a_rows, b_rows, 0);
     }
     return;
   }
@@ -417,25 +497,28 @@ __global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmParams p) {
   const int b_rows = (p.N - n0) < 256 ? (p.N - n0) : 256;
   const int k0 = ks * p.k_per_split;
   const int k_len = (p.K - k0) < p.k_per_split ? (p.K - k0) : p.k_per_split;
-  gemm_init_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows);
+  gemm_init_tile<T, OutT, kMContig>(p, acc, m0, n0, a_rows, b_rows);
 
-  constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;
   const int64_t s0 = k0 / Tile::kSlabK;   // first slab of this K range
   Tile::run(acc, Tile::Operand::blocked(static_cast<const T*>(p.A) + ((int64_t)mt * p.a_kslabs + s0) * kSlabElems, a_rows),
             Tile::Operand::blocked(static_cast<const T*>(p.B) + ((int64_t)nt * p.b_kslabs + s0) * kSlabElems, b_rows),
             k_len, lds);
-  gemm_store_tile<T, OutT>(p, acc, m0, n0, a_rows, b_rows, ks);
+  gemm_store_tile<T, OutT, kMContig>(p, acc, m0, n0, a_rows, b_rows, ks);
 }
 
-// C[m][n] (+)= sum over splits of partial[s][m][n]
+template <typename OutT> __device__ __forceinline__ OutT cvt_out(float v);
+template <> __device__ __forceinline__ float cvt_out<float>(float v) { return v; }
+template <> __device__ __forceinline__ __bf16 cvt_out<__bf16>(float v) { return (__bf16)v; }
+
+// C (+)= sum over splits of partial[s], each a dense copy of C's shape with `cols` elements per row
 template <typename OutT>
-__global__ void splitk_reduce_kernel(const float* __restrict__ partial, int k_split, int64_t MN, int N, OutT* C,
+__global__ void splitk_reduce_kernel(const float* __restrict__ partial, int k_split, int64_t MN, int cols, OutT* C,
                                      int64_t ldc, int accumulate) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < MN; i += (int64_t)gridDim.x * blockDim.x) {
     float v = 0.f;
     for (int s = 0; s < k_split; ++s) v += partial[(int64_t)s * MN + i];
-    const int64_t m = i / N, n = i - m * N;
-    OutT* dst = C + m * ldc + n;
+    const int64_t row = i / cols, col = i - row * cols;
+    OutT* dst = C + row * ldc + col;
     if (accumulate) v += (float)*dst;
     *dst = cvt_out<OutT>(v);
   }
@@ -522,12 +605,12 @@ static int pick_k_split(int tiles, int M, int N, int K, int slab, size_t partial
   return best;
 }
 
-template <typename T, typename OutT>
+template <typename T, typename OutT, bool kMContig>
 static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, int64_t b_kslabs, int N, int K, void* C,
                        int64_t ldc, int accumulate, hipStream_t stream, float* partial = nullptr,
                        size_t partial_bytes = 0) {
   using Tile = HeadTile<T>;
-  int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<T, OutT>), Tile::kLdsBytes, "gemm_nt_kernel");
+  int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<T, OutT, kMContig>), Tile::kLdsBytes, "gemm_nt_kernel");
   if (rc) return rc;
   GemmParams g;
   g.A = A; g.B = B; g.C = C; g.a_kslabs = a_kslabs; g.b_kslabs = b_kslabs; g.ldc = ldc;
@@ -538,20 +621,21 @@ static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, in
   g.k_split = partial ? pick_k_split(g.n_mt * g.n_nt, M, N, K, slab, partial_bytes) : 1;
   g.k_per_split = g.k_split > 1 ? (int)round_up64((K + g.k_split - 1) / g.k_split, slab) : K;
   g.partial = partial;
-  // Many more tiles than CUs and no K split: let 256 workgroups walk runs of m tiles instead of
+  // Many more tiles than CUs and no K split: let 256 workgroups walk runs of tiles instead of
   // launching one workgroup per tile.
+  const int n_fixed = kMContig ? g.n_mt : g.n_nt, n_moving = kMContig ? g.n_nt : g.n_mt;
   g.n_walk = 0;
-  if (g.k_split == 1 && g.n_nt <= 256 && g.n_mt * g.n_nt >= 4 * 256 && K >= 2 * slab) {
-    g.n_walk = 256 / g.n_nt;
-    if (g.n_walk > g.n_mt) g.n_walk = g.n_mt;
+  if (g.k_split == 1 && n_fixed <= 256 && g.n_mt * g.n_nt >= 4 * 256 && K >= 2 * slab) {
+    g.n_walk = 256 / n_fixed;
+    if (g.n_walk > n_moving) g.n_walk = n_moving;
   }
-  int grid = ((g.n_walk > 0 ? g.n_walk * g.n_nt : g.n_mt * g.n_nt * g.k_split) + 7) / 8 * 8;
-  hipLaunchKernelGGL((gemm_nt_kernel<T, OutT>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, g);
+  int grid = ((g.n_walk > 0 ? g.n_walk * n_fixed : g.n_mt * g.n_nt * g.k_split) + 7) / 8 * 8;
+  hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, kMContig>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, g);
   rc = check_launch("gemm_nt_kernel");
   if (rc || g.k_split == 1) return rc;
   const int64_t MN = (int64_t)M * N;
   int blocks = (int)((MN + 255) / 256 < 4096 ? (MN + 255) / 256 : 4096);
-  hipLaunchKernelGGL(splitk_reduce_kernel<OutT>, dim3(blocks), dim3(256), 0, stream, partial, g.k_split, MN, N,
+  hipLaunchKernelGGL(splitk_reduce_kernel<OutT>, dim3(blocks), dim3(256), 0, stream, partial, g.k_split, MN, kMContig ? M : N,
                      static_cast<OutT*>(C), ldc, accumulate);
   return check_launch("splitk_reduce_kernel");
 }
@@ -640,18 +724,18 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream, int64_t 
       if (rc) return rc;
     }
     if (a->dhidden) {
-      // dhidden[chunk][h] = sum_v dz[t][v] WT[h][v]
-      rc = launch_gemm<T, T>(dz, ldz / Tile::kSlabK, (int)tc, wt, pl.ldv / Tile::kSlabK, (int)H, (int)pl.ldv,
+      // dhidden[chunk][h] = sum_v WT[h][v] dz[t][v]   (M = H, N = tokens, C[n][m])
+      rc = launch_gemm<T, T, true>(wt, pl.ldv / Tile::kSlabK, (int)H, dz, ldz / Tile::kSlabK, (int)tc, (int)pl.ldv,
                              static_cast<T*>(a->dhidden) + c0 * H, H, 0, stream,
                              reinterpret_cast<float*>(ws + pl.off_part), pl.part_bytes);
       if (rc) return rc;
     }
     if (a->dweight) {
-      // hidT(h, t) = hidden[c0 + t][h], zero for tc <= t < ldt, K-blocked;  dW[v][h] (+)= sum_t dzT(v, t) hidT(h, t)
+      // hidT(h, t) = hidden[c0 + t][h], zero for tc <= t < ldt, K-blocked;  dW[v][h] (+)= sum_t dzT(v, t) hidT(h, t)   (M = V, N = H, C[m][n])
       rc = launch_transpose<T>(hidden + c0 * H, H, hidt, ldt, (int)tc, (int)H, stream);
       if (rc) return rc;
-      rc = launch_gemm<T, float>(dzt, ldt / Tile::kSlabK, (int)V, hidt, ldt / Tile::kSlabK, (int)H, (int)ldt, a->dweight, H,
-                                 (a->accumulate_dweight || c0 > 0) ? 1 : 0, stream);
+      rc = launch_gemm<T, float, false>(dzt, ldt / Tile::kSlabK, (int)V, hidt, ldt / Tile::kSlabK, (int)H, (int)ldt, a->dweight, H,
+                                        (a->accumulate_dweight || c0 > 0) ? 1 : 0, stream);
       if (rc) return rc;
     }
   }
