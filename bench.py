@@ -41,7 +41,7 @@ def build_workload(cfg, device):
     cu, mask = synthetic.packed_layout(samples)
     T = int(cu[-1])
     hidden, weight, labels = synthetic.make_head_tensors(cfg, T, gen, device=device, device_generate=True)
-    return samples, cu.to(device), mask.to(device), T, hidden, weight, labels
+    return samples, cu.to(device), mask.to(device), T, hidden, weight, labels, mask
 
 
 def advantages_for(samples, device):
@@ -293,7 +293,7 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     cfg = synthetic.CONFIGS[args.config]
-    samples, cu, mask, T, hidden, weight, labels = build_workload(cfg, dev)
+    samples, cu, mask, T, hidden, weight, labels, mask_host = build_workload(cfg, dev)
     train = cfg.loss is not None
     n_tok = float(mask.sum().item())
     adv = advantages_for(samples, dev)
@@ -335,7 +335,7 @@ def main():
                              entropy_coef=cfg.entropy_coef, temperature=cfg.temperature, dweight=dweight,
                              accumulate_dweight=False, keep_logits_chunk=keep, cu_seqlens_host=cu_host,
                              skip_masked_rows=not args.no_skip_masked, skip_masked_forward=args.skip_masked_forward,
-                             stage_hook=hook if record else None,
+                             stage_hook=hook if record else None, loss_mask_host=mask_host,
                              check_flags=False)
         if record:
             marks.append(cur)

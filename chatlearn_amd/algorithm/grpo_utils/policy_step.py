@@ -14,7 +14,7 @@ from typing import Any, Callable, Dict, List, Optional
 import torch
 
 from ... import ops
-from ...fused import grpo_head_step
+from ...fused import DEFAULT_KEEP_LOGITS_TOKENS, grpo_head_step
 from .trainer_utils import (batching, generate_loss_mask_position_ids, split_and_unpadding, split_microbatch,
                             unpad_input)
 
@@ -29,7 +29,7 @@ class PolicyStep:
                  module_args: Optional[Dict[str, Any]] = None, packing: bool = False, max_token_in_seq: int = 32768,
                  train_micro_batch_size: int = 1, generate_micro_batch_size: int = 1, trainable: bool = True,
                  fsdp_size: int = 1, temperature: float = 1.0, dweight_buffer: Optional[torch.Tensor] = None,
-                 keep_logits_chunk: Optional[int] = 16384):
+                 keep_logits_chunk: Optional[int] = DEFAULT_KEEP_LOGITS_TOKENS):
         self.backbone = backbone
         self.weight = lm_head_weight
         self.module_args = dict(_DEFAULT_ARGS)
@@ -93,22 +93,33 @@ class PolicyStep:
                 # labels roll along the (packed or padded) token row (policy_trainer.py:135,160)
                 labels, _ = ops.shift_labels(tokens.to(self.device).contiguous(), None, zero_last=False)
             # the training mask rolls along the padded rows and loses its last column (policy_trainer.py:161-162)
-            shifted = None
+            shifted = shifted_host = None
             if training:
                 _, shifted = ops.shift_labels(None, loss_mask.to(self.device).to(torch.int32).contiguous(),
                                               zero_last=True)
+                # the same shift on the host copy, flattened the way the kernels see the tokens: it tells the
+                # head step which rows carry a gradient without reading anything back from the device
+                shifted_host = torch.roll(loss_mask.cpu().to(torch.int32), shifts=-1, dims=1)
+                shifted_host[:, -1] = 0
+                if self.packing:
+                    lens = [p + r for p, r in zip(data_b["prompt_token_length"], data_b["response_token_length"])]
+                    shifted_host = torch.cat([shifted_host[i, :n] for i, n in enumerate(lens)])
+                else:
+                    shifted_host = shifted_host.reshape(-1)
             data_obj = {"all_tokens": tokens, "position_ids": position_ids, "labels": labels,
                         "ori_seq_len": ori_seq_len, "indices": indices, "cu_seqlens": cu_seqlens,
                         "ori_batch_size": ori_batch_size, "sample_ids": data_b["id_in_list"],
                         "attention_mask": attn_mask, "pad_size": 0}
             if training:
-                data_obj.update({"loss_mask": shifted, "old_logprobs": data_b["old_logprobs"],
+                data_obj.update({"loss_mask": shifted, "loss_mask_host": shifted_host,
+                                 "old_logprobs": data_b["old_logprobs"],
                                  "ref_logprobs": data_b["ref_logprobs"], "advantages": data_b["advantages"]})
             data_after_process.append(data_obj)
         return response_token_length_total, data_after_process
 
     def _to_device(self, inputs):
-        return {k: (v.to(self.device) if isinstance(v, torch.Tensor) else v) for k, v in inputs.items()}
+        return {k: (v.to(self.device) if isinstance(v, torch.Tensor) and not k.endswith("_host") else v)
+                for k, v in inputs.items()}
 
     def _flat_view(self, inputs, hidden):
         """hidden as [T, H] plus the per-token views of the padded [B, S] side inputs."""
@@ -148,7 +159,7 @@ class PolicyStep:
                 accumulate_dweight=accumulate, need_dhidden=flat.requires_grad,
                 keep_logits_chunk=self.keep_logits_chunk,
                 # only masked sums leave this method, so rows outside the loss mask need no forward either
-                skip_masked_forward=True, weight_t_cache=wt_cache)
+                skip_masked_forward=True, weight_t_cache=wt_cache, loss_mask_host=inputs["loss_mask_host"])
             dw, accumulate = out["dweight"], True
             if flat.requires_grad:
                 hidden.backward(out["dhidden"].reshape(hidden.shape))

@@ -20,14 +20,73 @@ from . import ops
 from ._lib import LOSS_GRPO, LOSS_GSPO
 
 
+DEFAULT_KEEP_LOGITS_TOKENS = 8192   # tokens whose logits one chunk keeps for its backward (2.5 GB at a 152k vocabulary)
+
+
 def _nonzero_rows(mask: torch.Tensor) -> torch.Tensor:
-    """Ascending positions of the nonzero entries of a flat int32 mask.  The index kernels use one
-    workgroup per row of a [B, S] mask, so the flat mask is presented as many short rows where its
-    length allows (the flat positions are the same)."""
+    """Ascending positions of the nonzero entries of a flat int32 device mask (one host round trip for
+    their count).  The index kernels use one workgroup per row of a [B, S] mask, so the flat mask is
+    presented as rows of 64 entries, zero-padded at the end (the flat positions are the same)."""
     n = mask.numel()
-    width = next((w for w in (256, 128, 64) if n % w == 0), n)
-    live, _, _, _ = ops.unpad_indices(mask.reshape(n // width, width))
+    if n == 0:
+        return torch.empty(0, dtype=torch.int64, device=mask.device)
+    if n % 64:
+        mask = torch.nn.functional.pad(mask, (0, 64 - n % 64))
+    live, _, _, _ = ops.unpad_indices(mask.reshape(-1, 64))
     return live
+
+
+class _PinnedStaging:
+    """Host-side staging for small index arrays that go to the device without stalling the host: two pinned
+    buffers used in turn, each guarded by an event so that it is not rewritten while its copy is in flight."""
+
+    def __init__(self):
+        self.slots = [None, None]
+        self.events = [None, None]
+        self.turn = 0
+
+    def upload(self, host: torch.Tensor, device) -> torch.Tensor:
+        i = self.turn
+        self.turn ^= 1
+        nbytes = host.numel() * host.element_size()
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        if self.slots[i] is None or self.slots[i].numel() < nbytes:
+            self.slots[i] = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, pin_memory=True)
+        stage = self.slots[i][:nbytes].view(host.dtype)
+        stage.copy_(host.reshape(-1))
+        out = stage.to(device, non_blocking=True)
+        self.events[i] = torch.cuda.Event()
+        self.events[i].record()
+        return out.reshape(host.shape)
+
+
+_staging = {}
+
+
+def _upload(host: torch.Tensor, device) -> torch.Tensor:
+    key = (torch.device(device).index or 0, host.dtype)
+    return _staging.setdefault(key, _PinnedStaging()).upload(host, device)
+
+
+def _live_rows_from_host_mask(mask_host: torch.Tensor, chunks, device):
+    """Per token chunk: (positions of the unmasked rows inside the chunk, int64; row map int32 with the
+    rank of each unmasked row or -1), built on the host from a host copy of the loss mask and sent
+    over in two asynchronous copies, so that no device value has to be read back."""
+    flat = mask_host.reshape(-1) != 0
+    live_all = torch.nonzero(flat).flatten()
+    bounds = torch.searchsorted(live_all, torch.tensor([lo for lo, _ in chunks] + [chunks[-1][1]]))
+    local = live_all.clone()
+    row_map = torch.full((flat.numel(),), -1, dtype=torch.int32)
+    counts = []
+    for k, (lo, hi) in enumerate(chunks):
+        a, b = int(bounds[k]), int(bounds[k + 1])
+        local[a:b] -= lo
+        row_map[live_all[a:b]] = torch.arange(b - a, dtype=torch.int32)
+        counts.append((a, b))
+    local_d = _upload(local, device) if local.numel() else torch.empty(0, dtype=torch.int64, device=device)
+    map_d = _upload(row_map, device)
+    return [(local_d[a:b], map_d[lo:hi]) for (a, b), (lo, hi) in zip(counts, chunks)]
 
 
 class _FusedHead(torch.autograd.Function):
@@ -98,7 +157,7 @@ class _FusedHead(torch.autograd.Function):
 def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, *,
                                  temperature: float = 1.0, need_entropy: bool = True,
                                  dweight_buffer: Optional[torch.Tensor] = None,
-                                 keep_logits_rows: Optional[int] = 16384, loss_mask: Optional[torch.Tensor] = None):
+                                 keep_logits_rows: Optional[int] = DEFAULT_KEEP_LOGITS_TOKENS, loss_mask: Optional[torch.Tensor] = None):
     """(logprob fp32 [T], entropy fp32 [T]) of ``labels`` under softmax(hidden @ weight.T / temperature).
 
     hidden [T,H] and weight [V,H] share a dtype (bf16 or fp32), labels int64 [T].
@@ -108,8 +167,11 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     Leading dimensions of hidden/labels are flattened and restored.
 
     ``keep_logits_rows``: when a gradient is needed and there are at most this many rows, the forward
-    keeps its raw logits (one copy in the input dtype, released by the backward) so that the backward
-    does not recompute them; ``None`` or more rows: recompute.  ``loss_mask`` (same shape as
+    keeps its raw logits (one 16-bit copy for 16-bit inputs, released by the backward) so that the
+    backward does not recompute them; ``None`` or more rows: recompute.  The default bounds the kept
+    logits at 2.5 GB for a 152k vocabulary; a caller that wants the fast path for a larger micro-batch
+    either raises it or runs the head chunk by chunk (forward, loss, backward per chunk), which is what
+    ``grpo_head_step`` does.  ``loss_mask`` (same shape as
     ``labels``) is a promise that rows where it is zero receive a zero upstream gradient - true
     of the reference's loss, which multiplies by this mask (policy_trainer.py:259-283): their
     logits are then not kept and the backward runs on the other rows only.
@@ -165,8 +227,9 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                    pos_clip_ratio=0.2, neg_clip_ratio=0.2, diff_clip_ratio=10, final_clip_ratio=3,
                    kl_coef=0.0, entropy_coef=0.0, temperature=1.0, dweight: Optional[torch.Tensor] = None,
                    accumulate_dweight=False, need_dhidden=True, check_flags=True,
-                   keep_logits_chunk: Optional[int] = 16384, cu_seqlens_host=None, skip_masked_rows=True,
-                   skip_masked_forward=False, weight_t_cache: Optional[dict] = None, stage_hook=None):
+                   keep_logits_chunk: Optional[int] = DEFAULT_KEEP_LOGITS_TOKENS, cu_seqlens_host=None,
+                   skip_masked_rows=True, skip_masked_forward=False, weight_t_cache: Optional[dict] = None,
+                   stage_hook=None, loss_mask_host: Optional[torch.Tensor] = None):
     """Forward + loss + backward of the head for one packed micro-batch, no autograd graph.
 
     Mirrors policy_trainer.py:216-286 on packed rows: returns a dict with the
@@ -191,6 +254,10 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     instead of the values the reference computes and then ignores; ``rows_projected_fwd`` counts
     the rows the forward ran on.
 
+    ``loss_mask_host``: a host copy of ``loss_mask`` (the trainer builds the mask on the host anyway).  With
+    it the unmasked rows of every chunk are found on the host and sent over asynchronously; without it
+    they are found on the device, which costs one host round trip per chunk for their count.
+
     ``weight_t_cache``: a dict the caller keeps while ``weight`` does not change (the micro-batches
     of one optimizer step).  The first backward leaves the transposed weight in it and later calls
     reuse it instead of transposing again; the caller clears it after updating the weight.
@@ -208,8 +275,23 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
         bounds = list(cu_seqlens_host) if cu_seqlens_host is not None else cu_seqlens.tolist()
     chunks = _token_chunks(T, keep_logits_chunk, bounds)
     zbuf = None
-    if keep_logits_chunk is not None:
-        zbuf = ops.saved_logits_buffer(max(hi - lo for lo, hi in chunks), V, hidden.dtype, hidden.device)
+    skip = keep_logits_chunk is not None and loss_mask is not None and skip_masked_rows
+    rows_of = None
+    if skip and loss_mask_host is not None and T > 0:
+        rows_of = _live_rows_from_host_mask(loss_mask_host, chunks, hidden.device)
+    longest = max(hi - lo for lo, hi in chunks)
+    if keep_logits_chunk is not None and T > 0:
+        kept = longest if rows_of is None else max(int(live.numel()) for live, _ in rows_of)
+        zbuf = ops.saved_logits_buffer(kept, V, hidden.dtype, hidden.device)
+    # scratch memory of the forward and the backward, shared by all chunks of this call
+    H = hidden.shape[1]
+    fwd_ws = torch.empty(max(ops.lmhead_forward_workspace_bytes(longest, H, V, hidden.dtype), 16), dtype=torch.uint8,
+                         device=hidden.device) if T > 0 else None
+    bwd_rows = longest if zbuf is None else min(longest, zbuf.shape[0])
+    bwd_ws = None
+    if zbuf is not None:
+        bwd_ws = torch.empty(ops.lmhead_backward_workspace_bytes(bwd_rows, H, V, hidden.dtype, True), dtype=torch.uint8,
+                             device=hidden.device)
     f = dict(dtype=torch.float32, device=hidden.device)
     lp_all, ent_all, lse_all, glp_all = (torch.empty(T, **f) for _ in range(4))
     loss_all = torch.empty(T, dtype=advantages.dtype, device=hidden.device)
@@ -228,29 +310,32 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
         wt = ops.weight_t_buffer(weight)
     kl_c = kl_coef if kl_coef > 0 else 0.0
     en_c = entropy_coef if entropy_coef > 0 else 0.0
-    for lo, hi in chunks:
+    for k, (lo, hi) in enumerate(chunks):
         sl = slice(lo, hi)
         n = hi - lo
         live = row_map = None
-        if zbuf is not None and loss_mask is not None and skip_masked_rows:
+        if skip and n > 0:
             # Rows whose loss mask is zero get a zero upstream gradient whatever the logits are:
             # keep logits only for the others and run the backward on that compact set of rows.
-            live = _nonzero_rows(loss_mask[sl])
-            row_map = torch.full((n,), -1, dtype=torch.int32, device=hidden.device)
-            row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
+            if rows_of is not None:
+                live, row_map = rows_of[k]
+            else:
+                live = _nonzero_rows(loss_mask[sl])
+                row_map = torch.full((n,), -1, dtype=torch.int32, device=hidden.device)
+                row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
         hook("forward")
         h_c = lab_c = None
         if live is not None and skip_masked_forward and live.numel() > 0:
             # forward on the compact set of unmasked rows; results scattered back, zeros elsewhere
             h_c, lab_c = ops.gather_rows(hidden[sl], live), ops.gather_rows(labels[sl].reshape(n, 1), live).reshape(-1)
             lp_c, ent_c, _, lse_c = ops.lmhead_forward(h_c, weight, lab_c, temperature, need_entropy=True,
-                                                       saved_logits=zbuf)
+                                                       saved_logits=zbuf, workspace=fwd_ws)
             spread = lambda x: ops.scatter_rows(x.reshape(-1, 1), live, n).reshape(-1)
             lp, ent, lse = spread(lp_c), spread(ent_c), spread(lse_c)
             rows_projected_fwd += int(live.numel())
         else:
             lp, ent, _, lse = ops.lmhead_forward(hidden[sl], weight, labels[sl], temperature, need_entropy=True,
-                                                 saved_logits=zbuf, saved_row_map=row_map)
+                                                 saved_logits=zbuf, saved_row_map=row_map, workspace=fwd_ws)
             rows_projected_fwd += n
         hook("loss")
         res = ops.policy_loss(
@@ -265,7 +350,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
             dh, dw = ops.lmhead_backward(hidden[sl], weight, labels[sl], lse, ent, res.g_logprob, res.g_entropy,
                                          temperature, need_dhidden=need_dhidden, need_dweight=True, dweight=dw,
                                          accumulate_dweight=acc_dw, saved_logits=zbuf, weight_t=wt,
-                                         weight_t_ready=wt_ready)
+                                         weight_t_ready=wt_ready, workspace=bwd_ws)
             wt_ready = True
         elif live.numel() == 0:
             dh = torch.zeros_like(hidden[sl]) if need_dhidden else None
@@ -281,7 +366,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                 h_c, weight, lab_c, pick(lse), pick(ent),
                 pick(res.g_logprob), pick(res.g_entropy), temperature, need_dhidden=need_dhidden,
                 need_dweight=True, dweight=dw, accumulate_dweight=acc_dw, saved_logits=zbuf, weight_t=wt,
-                weight_t_ready=wt_ready)
+                weight_t_ready=wt_ready, workspace=bwd_ws)
             wt_ready = True
             dh = ops.scatter_rows(dh_c, live, n) if need_dhidden else None
             rows_projected_bwd += int(live.numel()) - n

@@ -99,7 +99,7 @@ def weight_t_rowmajor(weight_t: torch.Tensor, H: int, V: int) -> torch.Tensor:
 def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[torch.Tensor],
                    temperature: float = 1.0, need_entropy: bool = True,
                    saved_logits: Optional[torch.Tensor] = None, saved_row_map: Optional[torch.Tensor] = None,
-                   _shard_begin: Optional[int] = None
+                   _shard_begin: Optional[int] = None, workspace: Optional[torch.Tensor] = None
                    ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], torch.Tensor, torch.Tensor]:
     """(logprob, entropy, rowmax, lse), each fp32 [T].  Logits are not materialised unless the caller
     hands in ``saved_logits`` (from ``saved_logits_buffer``) for these T rows, which a following
@@ -130,7 +130,8 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
         if T == 0:
             return logprob, entropy, rowmax, lse
     ws_bytes = _lib.lib().clgrpo_lmhead_fwd_workspace_bytes(T, H, V, dt)
-    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=hidden.device)
+    ws = workspace if (workspace is not None and workspace.numel() >= ws_bytes) else \
+        torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=hidden.device)
     ld_saved = 0
     if saved_logits is not None:
         saved_logits = _dev(saved_logits, "saved_logits", hidden.dtype)
@@ -153,6 +154,17 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
         return record
     _lib.call("clgrpo_lmhead_fwd", a, _stream(hidden))
     return logprob, entropy, rowmax, lse
+
+
+def lmhead_forward_workspace_bytes(T: int, H: int, V: int, dtype) -> int:
+    """Bytes of scratch one ``lmhead_forward`` call of T tokens needs."""
+    return int(_lib.lib().clgrpo_lmhead_fwd_workspace_bytes(T, H, V, BF16 if dtype == torch.bfloat16 else F32))
+
+
+def lmhead_backward_workspace_bytes(T: int, H: int, V: int, dtype, with_saved_logits: bool) -> int:
+    """Bytes of scratch one unchunked ``lmhead_backward`` call of T tokens needs."""
+    return int(_lib.lib().clgrpo_lmhead_bwd_workspace_bytes(T, H, V, BF16 if dtype == torch.bfloat16 else F32, T,
+                                                            1 if with_saved_logits else 0))
 
 
 def lmhead_forward_shard(hidden: torch.Tensor, weight_shard: torch.Tensor, labels: Optional[torch.Tensor],
@@ -198,7 +210,7 @@ def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=N
                     accumulate_dweight=False, chunk_tokens: Optional[int] = None,
                     max_workspace_bytes: int = DEFAULT_BWD_WORKSPACE_BYTES,
                     saved_logits: Optional[torch.Tensor] = None, weight_t: Optional[torch.Tensor] = None,
-                    weight_t_ready: bool = False, vocab_begin: int = 0):
+                    weight_t_ready: bool = False, vocab_begin: int = 0, workspace: Optional[torch.Tensor] = None):
     """(dhidden [T,H] in hidden's dtype, dweight [V,H] fp32).  ``dweight`` may be a caller
     buffer (e.g. the fp32 main-grad) that is overwritten or, with ``accumulate_dweight``, added to.
     ``saved_logits``: the buffer the forward of these rows filled; it is overwritten with d(logits).
@@ -256,7 +268,8 @@ def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=N
                 L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens, has_saved) > max_workspace_bytes:
             chunk_tokens = max(256, (chunk_tokens // 2 + 255) // 256 * 256)
     ws_bytes = L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens, has_saved)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=hidden.device)
+    ws = workspace if (workspace is not None and workspace.numel() >= ws_bytes) else \
+        torch.empty(ws_bytes, dtype=torch.uint8, device=hidden.device)
     a = _lib.LmheadBwdArgs(_ptr(hidden), _ptr(weight), _ptr(labels), _ptr(lse), _ptr(entropy), _ptr(g_logprob),
                            _ptr(g_entropy), T, H, V, dt, 1.0 / float(temperature), _ptr(dhidden), _ptr(dweight),
                            1 if accumulate_dweight else 0, _ptr(ws), ws.numel(), _ptr(saved_logits), ld_saved,

@@ -109,6 +109,25 @@ def test_head_step_matches_oracle(dev, name, kw, keep):
         assert_close_rel(got["dweight"], full["dweight"], 1e-5 if cfg.dtype == torch.float32 else 1e-2, "skip vs full dW")
 
 
+@pytest.mark.parametrize("keep", [512, 100000], ids=["chunked", "one-chunk"])
+def test_host_copy_of_the_loss_mask_gives_the_same_bits_without_reading_back(dev, keep):
+    """With a host copy of the loss mask the unmasked rows are found on the host (no device value is read
+    back); the results are bit-identical to the device-side search."""
+    from chatlearn_amd.fused import grpo_head_step
+    cfg, samples, cu, mask, T, hidden, weight, labels, old, ref, adv = _workload(CASES[1][0], dev, **CASES[1][1])
+    d = lambda x: x.to(dev)
+    args = [d(x) for x in (hidden, weight, labels, old, ref, adv, cu, mask)]
+    kw = dict(n_tokens_total=float(mask.sum()), kl_coef=cfg.kl_coef, entropy_coef=cfg.entropy_coef,
+              temperature=cfg.temperature, cu_seqlens_host=cu.tolist(), keep_logits_chunk=keep)
+    a = grpo_head_step(*args, **kw)
+    b = grpo_head_step(*args, loss_mask_host=mask, **kw)
+    for k in ("logprob", "entropy", "dhidden", "dweight", "sums", "g_logprob"):
+        assert torch.equal(a[k], b[k]), k
+    assert a["rows_projected_bwd"] == b["rows_projected_bwd"] == int(mask.sum())
+    lean = grpo_head_step(*args, loss_mask_host=mask, skip_masked_forward=True, **kw)
+    assert torch.equal(lean["dweight"], grpo_head_step(*args, skip_masked_forward=True, **kw)["dweight"])
+
+
 def test_kept_logits_backward_equals_recompute(dev):
     from chatlearn_amd import ops
     T, H, V = 700, 256, 5001
