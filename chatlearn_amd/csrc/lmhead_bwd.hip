@@ -561,7 +561,8 @@ struct BwdPlan {
   size_t off_wt, off_hidt, off_dz, off_dzt, off_part, part_bytes, total;
 };
 
-static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chunk_tokens, bool saved = false) {
+static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chunk_tokens, bool saved = false,
+                        bool own_wt = true) {
   BwdPlan pl;
   pl.ldv = round_up64(V, 64);
   int64_t chunk = (chunk_tokens <= 0 || chunk_tokens >= T) ? T : round_up64(chunk_tokens, 256);
@@ -571,7 +572,7 @@ static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chun
   size_t off = 0;
   // K-blocked operands: whole blocks of 256 rows
   const size_t Hb = (size_t)round_up64(H, 256), Cb = (size_t)round_up64(chunk, 256), Vb = (size_t)round_up64(V, 256);
-  pl.off_wt = off;   off += align_up(Hb * pl.ldv * es, 256);
+  pl.off_wt = off;   off += own_wt ? align_up(Hb * pl.ldv * es, 256) : 0;
   pl.off_hidt = off; off += align_up(Hb * pl.ldt * es, 256);
   pl.off_dz = off;   off += saved ? 0 : align_up(Cb * pl.ldv * es, 256);
   pl.off_dzt = off;  off += align_up(Vb * pl.ldt * es, 256);
@@ -582,12 +583,12 @@ static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chun
 }
 
 // Largest chunk (multiple of 256, or T itself) whose plan fits into `bytes`; 0 if none does.
-static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, size_t bytes, bool saved) {
-  if (bwd_plan(T, H, V, es, T, saved).total <= bytes) return T;
+static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, size_t bytes, bool saved, bool own_wt) {
+  if (bwd_plan(T, H, V, es, T, saved, own_wt).total <= bytes) return T;
   int64_t lo = 0, hi = T / 256;   // in units of 256 tokens
   while (lo < hi) {
     const int64_t mid = (lo + hi + 1) / 2;
-    if (bwd_plan(T, H, V, es, mid * 256, saved).total <= bytes) lo = mid; else hi = mid - 1;
+    if (bwd_plan(T, H, V, es, mid * 256, saved, own_wt).total <= bytes) lo = mid; else hi = mid - 1;
   }
   return lo * 256;
 }
@@ -652,11 +653,12 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream, int64_t 
   using Tile = HeadTile<T>;
   const int64_t T_ = a->T, H = a->H, V = a->V;
   const bool saved = a->saved_logits != nullptr;
-  const int64_t chunk = chunk_for_workspace(T_, H, V, sizeof(T), a->workspace_bytes, saved);
+  const bool own_wt = a->weight_t == nullptr;
+  const int64_t chunk = chunk_for_workspace(T_, H, V, sizeof(T), a->workspace_bytes, saved, own_wt);
   if (chunk <= 0)
     return fail(CLGRPO_EWORKSPACE, "clgrpo_lmhead_bwd: workspace %zu bytes cannot hold a 256-token chunk (%zu needed)",
-                a->workspace_bytes, bwd_plan(T_, H, V, sizeof(T), 256, saved).total);
-  const BwdPlan pl = bwd_plan(T_, H, V, sizeof(T), chunk, saved);
+                a->workspace_bytes, bwd_plan(T_, H, V, sizeof(T), 256, saved, own_wt).total);
+  const BwdPlan pl = bwd_plan(T_, H, V, sizeof(T), chunk, saved, own_wt);
   const int64_t ldz = saved ? a->ld_saved : pl.ldv;
   char* ws = static_cast<char*>(a->workspace);
   T* wt = a->weight_t ? static_cast<T*>(a->weight_t) : reinterpret_cast<T*>(ws + pl.off_wt);
@@ -749,7 +751,7 @@ using namespace clgrpo;
 extern "C" size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype,
                                                     int64_t chunk_tokens, int32_t with_saved_logits) {
   if (T <= 0 || H <= 0 || V <= 0 || (dtype != CLGRPO_BF16 && dtype != CLGRPO_F32)) return 0;
-  return bwd_plan(T, H, V, dtype_bytes(dtype), chunk_tokens, with_saved_logits != 0).total;
+  return bwd_plan(T, H, V, dtype_bytes(dtype), chunk_tokens, (with_saved_logits & 1) != 0, (with_saved_logits & 2) == 0).total;
 }
 
 static int bwd_entry(const char* who, const clgrpo_lmhead_bwd_args* a, int64_t vocab_begin, void* stream) {

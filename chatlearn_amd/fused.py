@@ -289,9 +289,6 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                          device=hidden.device) if T > 0 else None
     bwd_rows = longest if zbuf is None else min(longest, zbuf.shape[0])
     bwd_ws = None
-    if zbuf is not None:
-        bwd_ws = torch.empty(ops.lmhead_backward_workspace_bytes(bwd_rows, H, V, hidden.dtype, True), dtype=torch.uint8,
-                             device=hidden.device)
     f = dict(dtype=torch.float32, device=hidden.device)
     lp_all, ent_all, lse_all, glp_all = (torch.empty(T, **f) for _ in range(4))
     loss_all = torch.empty(T, dtype=advantages.dtype, device=hidden.device)
@@ -308,6 +305,9 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
         wt, wt_ready = weight_t_cache.get("weight_t"), weight_t_cache.get("weight_t") is not None
     if need_dhidden and wt is None and (len(chunks) > 1 or weight_t_cache is not None):
         wt = ops.weight_t_buffer(weight)
+    if zbuf is not None:
+        bwd_ws = torch.empty(ops.lmhead_backward_workspace_bytes(bwd_rows, H, V, hidden.dtype, True, wt is not None),
+                             dtype=torch.uint8, device=hidden.device)
     kl_c = kl_coef if kl_coef > 0 else 0.0
     en_c = entropy_coef if entropy_coef > 0 else 0.0
     for k, (lo, hi) in enumerate(chunks):
@@ -399,4 +399,12 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
             "entropy_loss_mean": en, "total_loss": total, "num_masked": sums[3],
             "per_token_loss": loss_all, "per_token_kl": kl_all, "dhidden": dh_all, "dweight": dw,
             "g_logprob": glp_all, "rows_projected_bwd": rows_projected_bwd,
-            "rows_projected_fwd": rows_projected_fwd, "sums": sums}
+            "rows_projected_fwd": rows_projected_fwd, "sums": sums,
+            # device memory this call held beyond its inputs and outputs: kept logits (they become d(logits) in
+            # place), the backward's operands (d(logits)^T, hidden^T, W^T unless the caller's cache holds it,
+            # split-K partials) and the forward's per-split records
+            "scratch_bytes": sum(t.numel() * t.element_size() for t in (zbuf, fwd_ws, bwd_ws) if t is not None)
+                             + (wt.numel() * wt.element_size() if wt is not None else 0)
+                             + (0 if (zbuf is not None or T == 0) else min(
+                                 ops.lmhead_backward_workspace_bytes(longest, H, V, hidden.dtype, False, wt is not None),
+                                 ops.DEFAULT_BWD_WORKSPACE_BYTES))}

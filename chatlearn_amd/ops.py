@@ -161,10 +161,11 @@ def lmhead_forward_workspace_bytes(T: int, H: int, V: int, dtype) -> int:
     return int(_lib.lib().clgrpo_lmhead_fwd_workspace_bytes(T, H, V, BF16 if dtype == torch.bfloat16 else F32))
 
 
-def lmhead_backward_workspace_bytes(T: int, H: int, V: int, dtype, with_saved_logits: bool) -> int:
+def lmhead_backward_workspace_bytes(T: int, H: int, V: int, dtype, with_saved_logits: bool,
+                                    caller_keeps_weight_t: bool = False) -> int:
     """Bytes of scratch one unchunked ``lmhead_backward`` call of T tokens needs."""
-    return int(_lib.lib().clgrpo_lmhead_bwd_workspace_bytes(T, H, V, BF16 if dtype == torch.bfloat16 else F32, T,
-                                                            1 if with_saved_logits else 0))
+    flags = (1 if with_saved_logits else 0) | (2 if caller_keeps_weight_t else 0)
+    return int(_lib.lib().clgrpo_lmhead_bwd_workspace_bytes(T, H, V, BF16 if dtype == torch.bfloat16 else F32, T, flags))
 
 
 def lmhead_forward_shard(hidden: torch.Tensor, weight_shard: torch.Tensor, labels: Optional[torch.Tensor],
@@ -262,12 +263,13 @@ def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=N
         weight_t = _dev(weight_t, "weight_t", hidden.dtype)
         if tuple(weight_t.shape) != (_round_up(H, 256), L.clgrpo_saved_logits_ld(V)) or not weight_t.is_contiguous():
             raise ValueError("weight_t must come from weight_t_buffer(weight)")
+    plan_flags = has_saved | (2 if weight_t is not None else 0)
     if chunk_tokens is None:
         chunk_tokens = T
         while chunk_tokens > 256 and \
-                L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens, has_saved) > max_workspace_bytes:
+                L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens, plan_flags) > max_workspace_bytes:
             chunk_tokens = max(256, (chunk_tokens // 2 + 255) // 256 * 256)
-    ws_bytes = L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens, has_saved)
+    ws_bytes = L.clgrpo_lmhead_bwd_workspace_bytes(T, H, V, dt, chunk_tokens, plan_flags)
     ws = workspace if (workspace is not None and workspace.numel() >= ws_bytes) else \
         torch.empty(ws_bytes, dtype=torch.uint8, device=hidden.device)
     a = _lib.LmheadBwdArgs(_ptr(hidden), _ptr(weight), _ptr(labels), _ptr(lse), _ptr(entropy), _ptr(g_logprob),

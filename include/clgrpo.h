@@ -117,8 +117,9 @@ typedef struct {
   int32_t weight_t_ready;   /* zero: this call fills weight_t; nonzero: it already holds W^T */
 } clgrpo_lmhead_bwd_args;
 
-/* Bytes needed to process `chunk_tokens` tokens at a time (chunk_tokens <= 0: all T at once);
- * with_saved_logits != 0: the d(logits) buffer is the caller's saved_logits, not part of the workspace. */
+/* Bytes needed to process `chunk_tokens` tokens at a time (chunk_tokens <= 0: all T at once).
+ * with_saved_logits is a bit set: bit 0: the d(logits) buffer is the caller's saved_logits, not part of the
+ * workspace; bit 1: the caller keeps W^T (weight_t), so the workspace holds no copy of it. */
 size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype,
                                          int64_t chunk_tokens, int32_t with_saved_logits);
 int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream);
