@@ -38,7 +38,8 @@ class LmheadBwdArgs(C.Structure):
                 ("g_logprob", vp), ("g_entropy", vp), ("T", i64), ("H", i64), ("V", i64),
                 ("dtype", i32), ("inv_temperature", f32), ("dhidden", vp), ("dweight", vp),
                 ("accumulate_dweight", i32), ("workspace", vp), ("workspace_bytes", sz),
-                ("saved_logits", vp), ("ld_saved", i64), ("weight_t", vp), ("weight_t_ready", i32)]
+                ("saved_logits", vp), ("ld_saved", i64), ("weight_t", vp), ("weight_t_ready", i32),
+                ("saved_rows", i64)]
 
 
 class SoftmaxStatsArgs(C.Structure):
@@ -48,7 +49,7 @@ class SoftmaxStatsArgs(C.Structure):
 
 class SoftmaxStatsBwdArgs(C.Structure):
     _fields_ = [("logits", vp), ("labels", vp), ("g_logprob", vp), ("g_entropy", vp), ("R", i64),
-                ("V", i64), ("ld", i64), ("dtype", i32), ("dlogits", vp)]
+                ("V", i64), ("ld", i64), ("dtype", i32), ("dlogits", vp), ("lse", vp), ("entropy", vp)]
 
 
 class PolicyLossArgs(C.Structure):

@@ -21,9 +21,11 @@ class _StatsFromLogits(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, logits2d, labels, want_lp, want_ent):
-        lp, ent, _ = ops.softmax_stats(logits2d, labels, need_entropy=want_ent, need_logprob=want_lp)
+        lp, ent, lse = ops.softmax_stats(logits2d, labels, need_entropy=want_ent, need_logprob=want_lp)
         ctx.set_materialize_grads(False)
-        ctx.save_for_backward(logits2d, labels if labels is not None else torch.empty(0, device=logits2d.device))
+        none = torch.empty(0, device=logits2d.device)
+        # the row statistics ride along (a few bytes per row) so that the backward reads each row once
+        ctx.save_for_backward(logits2d, labels if labels is not None else none, lse, ent if want_ent else none)
         ctx.want = (want_lp, want_ent)
         empty = torch.empty(0, device=logits2d.device)
         outs = (lp if want_lp else empty, ent if want_ent else empty)
@@ -35,13 +37,14 @@ class _StatsFromLogits(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_lp, g_ent):
-        logits2d, labels = ctx.saved_tensors
+        logits2d, labels, lse, ent = ctx.saved_tensors
         want_lp, want_ent = ctx.want
         g_lp = g_lp.float().contiguous() if (want_lp and g_lp is not None) else None
         g_ent = g_ent.float().contiguous() if (want_ent and g_ent is not None) else None
         if g_lp is None and g_ent is None:
             return None, None, None, None
-        return ops.softmax_stats_backward(logits2d, labels if g_lp is not None else None, g_lp, g_ent), None, None, None
+        return ops.softmax_stats_backward(logits2d, labels if g_lp is not None else None, g_lp, g_ent, lse=lse,
+                                          entropy=ent if g_ent is not None else None), None, None, None
 
 
 def _flatten_logits(logits):

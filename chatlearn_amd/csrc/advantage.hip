@@ -47,6 +47,13 @@ __global__ void group_advantage_kernel(clgrpo_group_advantage_args a) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= a.n_samples) return;
   const int g = a.group_of[i];
+  if (g < 0 || g >= a.n_groups) {
+    // a sample that names no group: NaN marks it instead of reading outside pool_offsets
+    a.advantages[i] = __longlong_as_double(0x7ff8000000000000LL);
+    if (a.all_zeros) a.all_zeros[i] = 0;
+    if (a.all_ones) a.all_ones[i] = 0;
+    return;
+  }
   const int lo = a.pool_offsets[g], hi = a.pool_offsets[g + 1];
   const double* x = a.pool + lo;
   const int n = hi - lo;

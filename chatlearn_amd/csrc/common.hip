@@ -49,6 +49,18 @@ int ensure_dynamic_lds(const void* kernel, int bytes, const char* name) {
   return CLGRPO_OK;
 }
 
+int device_cu_count() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+  cached[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
 }  // namespace clgrpo
 
 extern "C" int clgrpo_version(void) { return 100; }

@@ -13,6 +13,8 @@ int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
 // Raises the kernel's dynamic-LDS limit to `bytes` on the current device, once per (kernel, device).
 int ensure_dynamic_lds(const void* kernel, int bytes, const char* name);
+// Compute units of the current device (looked up once per device; 256 if the query fails).
+int device_cu_count();
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 inline int64_t round_up64(int64_t x, int64_t a) { return (x + a - 1) / a * a; }

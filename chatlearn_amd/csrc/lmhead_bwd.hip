@@ -593,14 +593,15 @@ static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, s
   return lo * 256;
 }
 
-// K ranges per tile that fill the 256 CUs best (1 = no split); at most what `partial_bytes` can hold.
+// K ranges per tile that fill the device's CUs best (1 = no split); at most what `partial_bytes` can hold.
 static int pick_k_split(int tiles, int M, int N, int K, int slab, size_t partial_bytes) {
+  const int cus = device_cu_count();
   int best = 1;
   double best_eff = 0.0;
   for (int s = 1; s <= 4; ++s) {
     if (s > 1 && ((size_t)s * M * N * sizeof(float) > partial_bytes || K / s < 8 * slab)) break;
     const long units = (long)tiles * s;
-    const double eff = (double)units / (double)(((units + 255) / 256) * 256);
+    const double eff = (double)units / (double)(((units + cus - 1) / cus) * cus);
     if (eff > best_eff + 0.04) { best_eff = eff; best = s; }   // a split must buy more than 4 % to be worth its extra pass
   }
   return best;
@@ -622,12 +623,13 @@ static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, in
   g.k_split = partial ? pick_k_split(g.n_mt * g.n_nt, M, N, K, slab, partial_bytes) : 1;
   g.k_per_split = g.k_split > 1 ? (int)round_up64((K + g.k_split - 1) / g.k_split, slab) : K;
   g.partial = partial;
-  // Many more tiles than CUs and no K split: let 256 workgroups walk runs of tiles instead of
+  // Many more tiles than CUs and no K split: let one workgroup per CU walk runs of tiles instead of
   // launching one workgroup per tile.
   const int n_fixed = kMContig ? g.n_mt : g.n_nt, n_moving = kMContig ? g.n_nt : g.n_mt;
+  const int cus = device_cu_count();
   g.n_walk = 0;
-  if (g.k_split == 1 && n_fixed <= 256 && g.n_mt * g.n_nt >= 4 * 256 && K >= 2 * slab) {
-    g.n_walk = 256 / n_fixed;
+  if (g.k_split == 1 && n_fixed <= cus && g.n_mt * g.n_nt >= 4 * cus && K >= 2 * slab) {
+    g.n_walk = cus / n_fixed;
     if (g.n_walk > n_moving) g.n_walk = n_moving;
   }
   int grid = ((g.n_walk > 0 ? g.n_walk * n_fixed : g.n_mt * g.n_nt * g.k_split) + 7) / 8 * 8;
@@ -771,6 +773,9 @@ static int bwd_entry(const char* who, const clgrpo_lmhead_bwd_args* a, int64_t v
   if (a->saved_logits != nullptr && (a->ld_saved < round_up64(a->V, 64) || a->ld_saved % 64 != 0))
     return fail(CLGRPO_ESHAPE, "%s: ld_saved=%lld must be a multiple of 64 and >= %lld", who, (long long)a->ld_saved,
                 (long long)round_up64(a->V, 64));
+  if (a->saved_logits != nullptr && a->saved_rows < round_up64(a->T, 256))
+    return fail(CLGRPO_ESHAPE, "%s: saved_rows=%lld, but the kept-logits buffer must hold %lld rows (T rounded up to 256)", who,
+                (long long)a->saved_rows, (long long)round_up64(a->T, 256));
   hipStream_t s = static_cast<hipStream_t>(stream);
   return a->dtype == CLGRPO_BF16 ? run_bwd<__bf16>(a, s, vocab_begin) : run_bwd<float>(a, s, vocab_begin);
 }

@@ -19,6 +19,7 @@ namespace clgrpo {
 
 constexpr int kFwdBM = 256, kFwdBN = 256;
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kMaxFwdSplits = 64;   // most vocabulary splits a forward launch uses
 
 struct FwdParams {
   const void* hidden;
@@ -294,16 +295,17 @@ __global__ void lmhead_fwd_finalize_kernel(FinalizeParams p) {
 }
 
 // Split of the vocabulary tiles over workgroups.  A workgroup walks ceil(n_vt / n_split) tiles for
-// one block of 256 tokens; with 256 CUs holding one workgroup each the launch takes
-// ceil(n_tb * n_split / 256) rounds, so the pick minimises rounds * tiles-per-workgroup.  At least
-// four splits when possible: the 32 workgroups of an XCD then form a 4 x 8 block sharing operands.
-static void fwd_plan(int64_t T, int64_t V, int& n_tb, int& n_vt, int& n_split, int& tiles_per_split) {
+// one block of 256 tokens; with each CU holding one workgroup the launch takes
+// ceil(n_tb * n_split / CUs) rounds, so the pick minimises rounds * tiles-per-workgroup.  At least
+// four splits when possible: the workgroups of an XCD then form a 4-row block sharing operands.
+// `cus` <= 0 plans for a 256-CU device (the workspace size must not depend on the device in use).
+static void fwd_plan(int64_t T, int64_t V, int& n_tb, int& n_vt, int& n_split, int& tiles_per_split, int cus = 0) {
   n_tb = (int)((T + kFwdBN - 1) / kFwdBN);
   n_vt = (int)((V + kFwdBM - 1) / kFwdBM);
-  const int cus = 256;
+  if (cus <= 0) cus = 256;
   int best = 1;
   long best_cost = -1;
-  for (int sp = 1; sp <= 64 && sp <= n_vt; ++sp) {
+  for (int sp = 1; sp <= kMaxFwdSplits && sp <= n_vt; ++sp) {
     const int tps = (n_vt + sp - 1) / sp;
     const int eff_sp = (n_vt + tps - 1) / tps;
     const long rounds = ((long)n_tb * eff_sp + cus - 1) / cus;
@@ -325,7 +327,7 @@ static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream, int64
   p.T = (int)a->T;
   p.H = (int)a->H;
   p.V = (int)a->V;
-  fwd_plan(a->T, a->V, p.n_tb, p.n_vt, p.n_split, p.tiles_per_split);
+  fwd_plan(a->T, a->V, p.n_tb, p.n_vt, p.n_split, p.tiles_per_split, device_cu_count());
   p.c = a->inv_temperature * kLog2e;
   p.part = static_cast<float4*>(a->workspace);
   p.z_out = a->saved_logits;
@@ -378,9 +380,11 @@ extern "C" size_t clgrpo_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_
   (void)H;
   (void)dtype;
   if (T <= 0 || V <= 0) return 0;
-  int n_tb, n_vt, n_split, tps;
-  fwd_plan(T, V, n_tb, n_vt, n_split, tps);
-  return (size_t)n_split * (size_t)T * sizeof(float4);
+  // one record per token and vocabulary split; the split count depends on the device's CU count and never
+  // exceeds kMaxFwdSplits, so this bound holds on any device
+  const int64_t n_vt = (V + kFwdBM - 1) / kFwdBM;
+  const int64_t splits = n_vt < kMaxFwdSplits ? n_vt : kMaxFwdSplits;
+  return (size_t)splits * (size_t)T * sizeof(float4);
 }
 
 // Shared by the whole-vocabulary entry point (record == nullptr) and the shard one.

@@ -6,11 +6,12 @@
 // step per block (+ a fixed-order pass over the per-block partials when more
 // than one block runs), so the sums are reproducible run to run.
 //
-// A micro-batch's worth of tokens (up to 2^18) goes through ONE launch of one
-// 1024-thread workgroup: sequence means (GSPO), per-token work, the reductions
-// and the flag word, with nothing to zero beforehand and no second pass.  The
-// work is a few hundred KB, so launch latency, not bandwidth, is what it costs.
-// Larger inputs take the multi-block kernels (sequence means, loss, finalize).
+// Up to 4096 tokens go through ONE launch of one 1024-thread workgroup: sequence
+// means (GSPO), per-token work, the reductions and the flag word.  Larger inputs
+// take the multi-block kernels: (sequence means,) the per-token pass, which leaves
+// per-block partial sums and flag bits, and a finalize pass that reduces them in a
+// fixed order - two launches (three for GSPO), nothing to zero beforehand.  The
+// work is a few hundred KB per micro-batch, so launch latency is what it costs.
 //
 // dtype rules follow what torch does in the reference: logprob arithmetic,
 // exp, clamp and the KL stay fp32; the product with the advantages (and the
@@ -24,7 +25,7 @@ constexpr int kLossThreads = 256;
 constexpr int kMaxLossBlocks = 1024;
 constexpr int kNumSums = 8;
 constexpr int kOneWgThreads = 1024;
-constexpr int64_t kOneWgMaxTokens = 1 << 18;   // above this the multi-block kernels take over
+constexpr int64_t kOneWgMaxTokens = 4096;   // above this the multi-block kernels take over
 
 struct LossParams {
   int mode;
@@ -219,12 +220,22 @@ __global__ __launch_bounds__(kLossThreads) void policy_loss_kernel(LossParams p)
     for (int k = 0; k < kNumSums; ++k) sh[threadIdx.x >> 6][k] = acc[k];
   }
   __syncthreads();
-  if (threadIdx.x < kNumSums) {
+  __shared__ int sh_flag[kLossThreads / 64];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) flag |= __shfl_xor(flag, off);
+  if ((threadIdx.x & 63) == 0) sh_flag[threadIdx.x >> 6] = flag;
+  __syncthreads();
+  if (threadIdx.x < kNumSums - 1) {
     double t = 0;
     for (int w = 0; w < kLossThreads / 64; ++w) t += sh[w][threadIdx.x];
     p.partials[(int64_t)blockIdx.x * kNumSums + threadIdx.x] = t;
   }
-  if (flag) atomicOr(p.flags, flag);
+  if (threadIdx.x == kNumSums - 1) {
+    // the last slot (always zero in the sums) carries this block's flag bits to the finalize pass
+    int f = 0;
+    for (int w = 0; w < kLossThreads / 64; ++w) f |= sh_flag[w];
+    p.partials[(int64_t)blockIdx.x * kNumSums + threadIdx.x] = (double)f;
+  }
 }
 
 
@@ -277,15 +288,21 @@ __global__ __launch_bounds__(kOneWgThreads) void policy_loss_onewg_kernel(LossPa
   }
 }
 
-__global__ void policy_loss_finalize_kernel(const double* partials, int n_blocks, double* sums) {
+// Fixed-order pass over the per-block partials: the sums, and the flag word OR-ed from the blocks' flag slots.
+__global__ void policy_loss_finalize_kernel(const double* partials, int n_blocks, double* sums, int32_t* flags) {
   const int k = threadIdx.x;
   if (k >= kNumSums) return;
+  if (k == kNumSums - 1) {
+    int f = 0;
+    for (int b = 0; b < n_blocks; ++b) f |= (int)partials[(int64_t)b * kNumSums + k];
+    flags[0] = f;
+    sums[k] = 0.0;
+    return;
+  }
   double t = 0;
   for (int b = 0; b < n_blocks; ++b) t += partials[(int64_t)b * kNumSums + k];
   sums[k] = t;
 }
-
-__global__ void zero_flags_kernel(int32_t* flags) { flags[0] = 0; }
 
 // Masked sums of up to kMaxMaskedSums per-token tensors in one launch of one workgroup (fixed
 // summation order): out[j] = sum_i float(src_j[i]) * mask[i], divided by (1e-5 + sum(mask)) where
@@ -415,7 +432,6 @@ static int run_policy_loss(const char* who, const clgrpo_policy_loss_args* a, vo
       hipLaunchKernelGGL(policy_loss_onewg_kernel<double>, dim3(1), dim3(kOneWgThreads), 0, s, p);
     return check_launch("policy_loss_onewg_kernel");
   }
-  hipLaunchKernelGGL(zero_flags_kernel, dim3(1), dim3(1), 0, s, a->flags);
   if (a->mode == CLGRPO_LOSS_GSPO) {
     hipLaunchKernelGGL(gspo_seq_mean_kernel, dim3((unsigned)a->B), dim3(kLossThreads), 0, s, p);
     int rc = check_launch("gspo_seq_mean_kernel");
@@ -428,7 +444,7 @@ static int run_policy_loss(const char* who, const clgrpo_policy_loss_args* a, vo
     hipLaunchKernelGGL(policy_loss_kernel<double>, dim3(blocks), dim3(kLossThreads), 0, s, p);
   int rc = check_launch("policy_loss_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL(policy_loss_finalize_kernel, dim3(1), dim3(64), 0, s, p.partials, blocks, a->sums);
+  hipLaunchKernelGGL(policy_loss_finalize_kernel, dim3(1), dim3(64), 0, s, p.partials, blocks, a->sums, a->flags);
   return check_launch("policy_loss_finalize_kernel");
 }
 
@@ -484,7 +500,7 @@ extern "C" int clgrpo_policy_loss_static(const clgrpo_policy_loss_args* a, void*
 
 extern "C" int clgrpo_policy_loss_launches(int64_t n, int32_t mode) {
   if (n <= kOneWgMaxTokens) return 1;
-  return mode == CLGRPO_LOSS_GSPO ? 4 : 3;
+  return mode == CLGRPO_LOSS_GSPO ? 3 : 2;
 }
 
 extern "C" int clgrpo_masked_sums(const clgrpo_masked_sums_args* a, void* stream) {

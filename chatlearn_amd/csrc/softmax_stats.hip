@@ -1,8 +1,9 @@
 // Softmax statistics (logprob, entropy, lse) from materialised logits and the
 // matching d(logits), for call sites that already hold [R, V] logits.
-// One 256-thread block per row; the row is streamed once for the statistics
-// (online max / sum / weighted sum, fp32) and, in the backward, once more to
-// write d(logits).  HBM-bound: V*sizeof(dtype) bytes per row read (+ written).
+// One 256-thread block per row, 16 bytes per lane and four loads in flight per thread; the row is
+// streamed once for the statistics (online max / sum / weighted sum, fp32).  The backward reads
+// it once more and writes d(logits), taking lse / entropy from the forward when the caller kept
+// them.  HBM-bound: V*sizeof(dtype) bytes per row read (+ the same written).
 #include "common.hpp"
 
 namespace clgrpo {
@@ -22,20 +23,78 @@ __device__ __forceinline__ void rs_merge(RowStats& a, const RowStats& b) {
   a.m = nm;
 }
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// 16 bytes of a row as floats.
+template <typename T> struct Vec16 {
+  static constexpr int N = 16 / (int)sizeof(T);
+  __device__ static __forceinline__ void unpack(const u32x4_t& raw, float (&z)[N]) {
+    const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int k = 0; k < N; ++k) z[k] = to_f32<T>(e[k]);
+  }
+  __device__ static __forceinline__ u32x4_t pack(const float (&d)[N]) {
+    alignas(16) T e[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) e[k] = (T)d[k];
+    return *reinterpret_cast<const u32x4_t*>(e);
+  }
+};
+
+// Online (max, sum e^{z-max}, sum e^{z-max} z) update with N new values: one rescale, then N exponentials
+// against a fixed maximum (no per-element branch).
+template <int N>
+__device__ __forceinline__ void rs_update(RowStats& st, const float (&z)[N]) {
+  float vmax = z[0];
+#pragma unroll
+  for (int k = 1; k < N; ++k) vmax = fmaxf(vmax, z[k]);
+  if (vmax > st.m) {
+    const float f = expf(st.m - vmax);   // st.m = -inf -> 0
+    st.s *= f;
+    st.u *= f;
+    st.m = vmax;
+  }
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    const float e = expf(z[k] - st.m);
+    st.s += e;
+    st.u = fmaf(e, z[k], st.u);
+  }
+}
+
+// Rows whose start and length are multiples of 16 bytes are streamed 16 bytes per lane, four
+// independent loads in flight per thread; other rows element by element.
 template <typename T>
-__device__ RowStats row_stats(const T* row, int64_t V) {
+__device__ __forceinline__ bool rows_vectorizable(const void* base, int64_t ld, int64_t V) {
+  constexpr int N = Vec16<T>::N;
+  return (reinterpret_cast<uintptr_t>(base) % 16 == 0) && (ld % N == 0) && (V % N == 0);
+}
+
+template <typename T>
+__device__ RowStats row_stats(const T* row, int64_t V, bool vec) {
+  constexpr int N = Vec16<T>::N;
   RowStats st{-INFINITY, 0.f, 0.f};
-  for (int64_t v = threadIdx.x; v < V; v += 256) {
-    const float z = to_f32<T>(row[v]);
-    if (z > st.m) {
-      const float f = expf(st.m - z);   // st.m = -inf -> 0
-      st.s = st.s * f + 1.f;
-      st.u = st.u * f + z;
-      st.m = z;
-    } else {
-      const float e = expf(z - st.m);
-      st.s += e;
-      st.u = fmaf(e, z, st.u);
+  if (vec) {
+    const u32x4_t* rv = reinterpret_cast<const u32x4_t*>(row);
+    const int64_t nvec = V / N;
+    int64_t i = threadIdx.x;
+    for (; i + 3 * 256 < nvec; i += 4 * 256) {
+      const u32x4_t r0 = rv[i], r1 = rv[i + 256], r2 = rv[i + 512], r3 = rv[i + 768];
+      float z[N];
+      Vec16<T>::unpack(r0, z); rs_update<N>(st, z);
+      Vec16<T>::unpack(r1, z); rs_update<N>(st, z);
+      Vec16<T>::unpack(r2, z); rs_update<N>(st, z);
+      Vec16<T>::unpack(r3, z); rs_update<N>(st, z);
+    }
+    for (; i < nvec; i += 256) {
+      float z[N];
+      Vec16<T>::unpack(rv[i], z);
+      rs_update<N>(st, z);
+    }
+  } else {
+    for (int64_t v = threadIdx.x; v < V; v += 256) {
+      const float z[1] = {to_f32<T>(row[v])};
+      rs_update<1>(st, z);
     }
   }
   for (int off = 32; off > 0; off >>= 1) {
@@ -57,7 +116,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void softmax_stats_kernel(clgrpo_softmax_stats_args a) {
   const int64_t r = blockIdx.x;
   const T* row = static_cast<const T*>(a.logits) + r * a.ld;
-  const RowStats st = row_stats<T>(row, a.V);
+  const RowStats st = row_stats<T>(row, a.V, rows_vectorizable<T>(a.logits, a.ld, a.V));
   if (threadIdx.x == 0) {
     const float lse = st.m + logf(st.s);
     if (a.lse) a.lse[r] = lse;
@@ -69,24 +128,53 @@ __global__ __launch_bounds__(256) void softmax_stats_kernel(clgrpo_softmax_stats
   }
 }
 
+// d(logits) of one row: with the row's lse (and entropy, when it carries a gradient) from the forward the
+// row is read once and written once; without them the statistics are rebuilt by one more pass over it.
 template <typename T>
 __global__ __launch_bounds__(256) void softmax_stats_bwd_kernel(clgrpo_softmax_stats_bwd_args a) {
+  constexpr int N = Vec16<T>::N;
   const int64_t r = blockIdx.x;
   const T* row = static_cast<const T*>(a.logits) + r * a.ld;
   T* out = static_cast<T*>(a.dlogits) + r * a.V;
-  const RowStats st = row_stats<T>(row, a.V);
-  const float lse = st.m + logf(st.s);
-  const float ent = lse - st.u / st.s;
+  const bool vec = rows_vectorizable<T>(a.logits, a.ld, a.V) && (reinterpret_cast<uintptr_t>(a.dlogits) % 16 == 0);
+  float lse, ent;
+  if (a.lse != nullptr && (a.g_entropy == nullptr || a.entropy != nullptr)) {
+    lse = a.lse[r];
+    ent = a.g_entropy ? a.entropy[r] : 0.f;
+  } else {
+    const RowStats st = row_stats<T>(row, a.V, vec);
+    lse = st.m + logf(st.s);
+    ent = lse - st.u / st.s;
+  }
   const float glp = a.g_logprob ? a.g_logprob[r] : 0.f;
   const float gen = a.g_entropy ? a.g_entropy[r] : 0.f;
   const int64_t y = a.g_logprob ? a.labels[r] : -1;
-  for (int64_t v = threadIdx.x; v < a.V; v += 256) {
-    const float z = to_f32<T>(row[v]);
+  auto dz = [&](float z, int64_t v) {
     const float logp = z - lse;
     const float p = expf(logp);
     float d = -p * (glp + gen * (logp + ent));
     if (v == y) d += glp;
-    out[v] = (T)d;
+    return d;
+  };
+  if (vec) {
+    const u32x4_t* rv = reinterpret_cast<const u32x4_t*>(row);
+    u32x4_t* ov = reinterpret_cast<u32x4_t*>(out);
+    const int64_t nvec = a.V / N;
+    auto one = [&](const u32x4_t& raw, int64_t i) {
+      float z[N], d[N];
+      Vec16<T>::unpack(raw, z);
+#pragma unroll
+      for (int k = 0; k < N; ++k) d[k] = dz(z[k], i * N + k);
+      ov[i] = Vec16<T>::pack(d);
+    };
+    int64_t i = threadIdx.x;
+    for (; i + 3 * 256 < nvec; i += 4 * 256) {
+      const u32x4_t r0 = rv[i], r1 = rv[i + 256], r2 = rv[i + 512], r3 = rv[i + 768];
+      one(r0, i); one(r1, i + 256); one(r2, i + 512); one(r3, i + 768);
+    }
+    for (; i < nvec; i += 256) one(rv[i], i);
+  } else {
+    for (int64_t v = threadIdx.x; v < a.V; v += 256) out[v] = (T)dz(to_f32<T>(row[v]), v);
   }
 }
 

@@ -275,7 +275,8 @@ def lmhead_backward(hidden, weight, labels, lse, entropy, g_logprob, g_entropy=N
     a = _lib.LmheadBwdArgs(_ptr(hidden), _ptr(weight), _ptr(labels), _ptr(lse), _ptr(entropy), _ptr(g_logprob),
                            _ptr(g_entropy), T, H, V, dt, 1.0 / float(temperature), _ptr(dhidden), _ptr(dweight),
                            1 if accumulate_dweight else 0, _ptr(ws), ws.numel(), _ptr(saved_logits), ld_saved,
-                           _ptr(weight_t), 1 if (weight_t is not None and weight_t_ready) else 0)
+                           _ptr(weight_t), 1 if (weight_t is not None and weight_t_ready) else 0,
+                           saved_logits.shape[0] if saved_logits is not None else 0)
     if vocab_begin:
         _lib.check(L.clgrpo_lmhead_bwd_shard(_lib.C.byref(a), int(vocab_begin), _lib.vp(_stream(hidden) or 0)))
     else:
@@ -309,7 +310,9 @@ def softmax_stats(logits2d: torch.Tensor, labels: Optional[torch.Tensor], need_e
     return lp, ent, lse
 
 
-def softmax_stats_backward(logits2d, labels, g_logprob, g_entropy):
+def softmax_stats_backward(logits2d, labels, g_logprob, g_entropy, lse=None, entropy=None):
+    """d(logits) [R,V] in the logits' dtype.  ``lse`` (and ``entropy`` when ``g_entropy`` is given) from the
+    forward let the kernel read each row once; without them it rebuilds them with one more pass."""
     if not logits2d.is_cuda:
         raise RuntimeError("logits must live on the GPU; this package has no CPU path")
     if logits2d.stride(1) != 1:
@@ -322,8 +325,12 @@ def softmax_stats_backward(logits2d, labels, g_logprob, g_entropy):
         labels = _dev(labels, "labels", torch.int64)
     if g_entropy is not None:
         g_entropy = _dev(g_entropy, "g_entropy", torch.float32)
+    if lse is not None:
+        lse = _dev(lse, "lse", torch.float32)
+    if entropy is not None:
+        entropy = _dev(entropy, "entropy", torch.float32)
     a = _lib.SoftmaxStatsBwdArgs(_ptr(logits2d), _ptr(labels) if g_logprob is not None else None, _ptr(g_logprob),
-                                 _ptr(g_entropy), R, V, ld, _dtype_enum(logits2d), _ptr(out))
+                                 _ptr(g_entropy), R, V, ld, _dtype_enum(logits2d), _ptr(out), _ptr(lse), _ptr(entropy))
     _lib.call("clgrpo_softmax_stats_bwd", a, _stream(logits2d))
     return out
 

@@ -115,6 +115,8 @@ typedef struct {
                                rows of clgrpo_saved_logits_ld(V) elements), so that several calls with the same
                                weight (token chunks of one step) build it once */
   int32_t weight_t_ready;   /* zero: this call fills weight_t; nonzero: it already holds W^T */
+  int64_t saved_rows;       /* rows the saved_logits buffer holds; must be >= ceil(T / 256) * 256 (the backward
+                               rewrites whole 256-row units) */
 } clgrpo_lmhead_bwd_args;
 
 /* Bytes needed to process `chunk_tokens` tokens at a time (chunk_tokens <= 0: all T at once).
@@ -174,6 +176,9 @@ typedef struct {
   int64_t R, V, ld;
   int32_t dtype;
   void* dlogits;           /* [R, V] out, `dtype`, row stride V */
+  const float* lse;        /* [R] from clgrpo_softmax_stats, or NULL: the row statistics are then rebuilt by one
+                              more pass over the logits */
+  const float* entropy;    /* [R] from clgrpo_softmax_stats; used (with lse) when g_entropy != NULL */
 } clgrpo_softmax_stats_bwd_args;
 int clgrpo_softmax_stats_bwd(const clgrpo_softmax_stats_bwd_args* a, void* stream);
 
@@ -226,8 +231,9 @@ typedef struct {
 
 size_t clgrpo_policy_loss_workspace_bytes(int64_t n, int64_t B);
 int clgrpo_policy_loss(const clgrpo_policy_loss_args* a, void* stream);
-/* Kernel launches one clgrpo_policy_loss call of n tokens enqueues (1 up to 2^18 tokens: sequence
- * means, per-token pass, sums and flag word run in a single workgroup). */
+/* Kernel launches one clgrpo_policy_loss call of n tokens enqueues: 1 up to 4096 tokens (sequence means,
+ * per-token pass, sums and flag word in a single workgroup), else 2 (per-token pass, finalize) plus 1 for
+ * the sequence means of CLGRPO_LOSS_GSPO. */
 int clgrpo_policy_loss_launches(int64_t n, int32_t mode);
 
 /* clgrpo_policy_loss without a workspace and without any allocation.  No counterpart in the reference: it

@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 def test_struct_sizes_match_header_layout():
     # 64-bit pointers and int64 fields, natural alignment
     assert C.sizeof(_lib.LmheadFwdArgs) == 3 * 8 + 3 * 8 + 4 + 4 + 4 * 8 + 8 + 8 + 8 + 8 + 8 + 8
-    assert C.sizeof(_lib.LmheadBwdArgs) == 7 * 8 + 3 * 8 + 4 + 4 + 2 * 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8
+    assert C.sizeof(_lib.LmheadBwdArgs) == 7 * 8 + 3 * 8 + 4 + 4 + 2 * 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8 + 8
     assert C.sizeof(_lib.RowsArgs) == 6 * 8
     assert C.sizeof(_lib.MaskedSumsArgs) == 8 + 8 + 16 * 8 + 16 * 4 + 16 * 4 + 3 * 8
 
@@ -49,7 +49,10 @@ def test_validation_before_launch(lib):
     a.dtype = _lib.BF16
     assert lib.clgrpo_lmhead_fwd(C.byref(a), None) == -4 and "hidden" in _err(lib)          # ENULL
     assert lib.clgrpo_lmhead_fwd(None, None) == -4
-    assert lib.clgrpo_lmhead_fwd_workspace_bytes(16384, 4096, 151936, _lib.BF16) == 4 * 16384 * 16
+    # one 16-byte record per token and vocabulary split, at most 64 splits whatever the device's CU count
+    assert lib.clgrpo_lmhead_fwd_workspace_bytes(16384, 4096, 151936, _lib.BF16) == 64 * 16384 * 16
+    assert lib.clgrpo_lmhead_fwd_workspace_bytes(100, 128, 700, _lib.BF16) == 3 * 100 * 16          # 3 vocabulary tiles
+    wt_kept = lib.clgrpo_lmhead_bwd_workspace_bytes(1024, 128, 1000, _lib.BF16, 0, 3)
     b = _lib.LmheadBwdArgs()
     b.T, b.H, b.V, b.dtype = 8, 128, 50, _lib.F32
     assert lib.clgrpo_lmhead_bwd(C.byref(b), None) == -4
@@ -57,6 +60,7 @@ def test_validation_before_launch(lib):
     half = lib.clgrpo_lmhead_bwd_workspace_bytes(1024, 128, 1000, _lib.BF16, 512, 0)
     saved = lib.clgrpo_lmhead_bwd_workspace_bytes(1024, 128, 1000, _lib.BF16, 0, 1)
     assert 0 < half < full and saved == full - 1024 * 1024 * 2   # minus the [T][ld] d(logits) buffer
+    assert wt_kept == saved - 256 * 1024 * 2                       # minus the workspace's own W^T (H rounded up to 256 rows)
     assert lib.clgrpo_saved_logits_ld(151936) == 151936 and lib.clgrpo_saved_logits_ld(1000) == 1024
     p = _lib.PolicyLossArgs()
     p.mode = 5

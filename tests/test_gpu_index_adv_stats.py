@@ -142,11 +142,12 @@ def test_group_advantage_large_pool_and_flags(dev):
     assert (got[-8:] == 0).all()
 
 
+@pytest.mark.parametrize("V", [1999, 6000], ids=["odd-V-elementwise", "V-16-byte-rows"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_stats_from_logits_mirrors(dev, dtype):
+def test_stats_from_logits_mirrors(dev, dtype, V):
     from chatlearn_amd.algorithm.grpo_utils import trainer_utils as tu
     g = torch.Generator().manual_seed(4)
-    B, S, V = 2, 300, 1999
+    B, S = 2, 300
     logits = (torch.randn(B, S, V, generator=g) * 2).to(dtype)
     labels = torch.randint(0, V, (B, S), generator=g)
     z64 = logits.double()
@@ -168,3 +169,16 @@ def test_stats_from_logits_mirrors(dev, dtype):
     # a strided view along the row dimension (what slicing logits[:, a:b] produces)
     part = ld.detach()[:, 10:50]
     assert_close_rel(tu.entropy_from_logits_with_chunking(part), osm.entropy_from_logits(z64[:, 10:50]), rt, "slice")
+    # a view whose rows are wider than the vocabulary slice it exposes (row stride > V), and the backward
+    # without the forward's statistics (the kernel rebuilds them) giving the same d(logits)
+    from chatlearn_amd import ops
+    wide = ld.detach().reshape(B * S, V)
+    half = wide[:, : (V // 16) * 8]
+    lp_h, en_h, lse_h = ops.softmax_stats(half, labels.reshape(-1).to(dev) % half.shape[1])
+    assert_close_rel(en_h, osm.entropy_from_logits(z64.reshape(B * S, V)[:, : half.shape[1]]), rt, "strided rows")
+    gl = w1.reshape(-1).to(dev)
+    ge = w2.reshape(-1).to(dev)
+    lab_h = labels.reshape(-1).to(dev) % half.shape[1]
+    d_with = ops.softmax_stats_backward(half, lab_h, gl, ge, lse=lse_h, entropy=en_h)
+    d_without = ops.softmax_stats_backward(half, lab_h, gl, ge)
+    assert_close_rel(d_with, d_without, 1e-5 if dtype == torch.float32 else 2 ** -7, "backward with / without kept statistics")
