@@ -680,6 +680,7 @@ def main():
     if train and not args.no_variants:
         out["gemm_kernels"] = gemm_kernels(w, keep)
         out["loss_stage"] = loss_stage(w)
+        torch.cuda.empty_cache()
         variants = {}
         plan = [("chunk_4096", dict(keep=4096)), ("whole_micro_batch_kept", dict(keep=T)),
                 ("recompute_no_logits_kept", dict(keep=None)),
@@ -687,7 +688,8 @@ def main():
                 ("skip_masked_rows_in_forward_too", dict(keep=keep, skip_masked_forward=True))]
         for name, kw in plan:
             k = kw.pop("keep")
-            v_dt, v_st, v_out = time_step(w, k, dweight, max(3, args.steps // 2), 2, **kw)
+            torch.cuda.empty_cache()     # each variant sizes its scratch differently: start from an unfragmented pool
+            v_dt, v_st, v_out = time_step(w, k, dweight, max(3, args.steps // 2), 3, **kw)
             variants[name] = step_record(w, k, v_dt, v_st, v_out)
         variants["note"] = ("same micro-batch; chunk_4096 / whole_micro_batch_kept: other chunk sizes of the kept logits; "
                             "recompute: nothing kept, logit tiles recomputed in the backward; no_row_skipping: backward on all T rows; "
@@ -709,6 +711,7 @@ def main():
     if args.autograd_seam and train:
         out["autograd_seam"] = autograd_seam(w, max(2, args.steps // 2))
     if train and not args.no_sweep:
+        torch.cuda.empty_cache()
         out["sweep"] = sweep(cfg, dev, w.weight, keep)
     if not args.no_other_configs:
         del w, dweight, out_last

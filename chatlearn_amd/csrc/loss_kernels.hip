@@ -288,20 +288,23 @@ __global__ __launch_bounds__(kOneWgThreads) void policy_loss_onewg_kernel(LossPa
   }
 }
 
-// Fixed-order pass over the per-block partials: the sums, and the flag word OR-ed from the blocks' flag slots.
+// Fixed-order pass over the per-block partials: one wavefront per sum (lane l adds blocks l, l + 64, ...,
+// then a shuffle tree), and the flag word OR-ed from the blocks' flag slots.  Launched with kNumSums * 64 threads.
 __global__ void policy_loss_finalize_kernel(const double* partials, int n_blocks, double* sums, int32_t* flags) {
-  const int k = threadIdx.x;
+  const int k = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (k >= kNumSums) return;
   if (k == kNumSums - 1) {
     int f = 0;
-    for (int b = 0; b < n_blocks; ++b) f |= (int)partials[(int64_t)b * kNumSums + k];
-    flags[0] = f;
-    sums[k] = 0.0;
+    for (int b = lane; b < n_blocks; b += 64) f |= (int)partials[(int64_t)b * kNumSums + k];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) f |= __shfl_xor(f, off);
+    if (lane == 0) { flags[0] = f; sums[k] = 0.0; }
     return;
   }
   double t = 0;
-  for (int b = 0; b < n_blocks; ++b) t += partials[(int64_t)b * kNumSums + k];
-  sums[k] = t;
+  for (int b = lane; b < n_blocks; b += 64) t += partials[(int64_t)b * kNumSums + k];
+  t = wave_sum(t);
+  if (lane == 0) sums[k] = t;
 }
 
 // Masked sums of up to kMaxMaskedSums per-token tensors in one launch of one workgroup (fixed
@@ -444,7 +447,7 @@ static int run_policy_loss(const char* who, const clgrpo_policy_loss_args* a, vo
     hipLaunchKernelGGL(policy_loss_kernel<double>, dim3(blocks), dim3(kLossThreads), 0, s, p);
   int rc = check_launch("policy_loss_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL(policy_loss_finalize_kernel, dim3(1), dim3(64), 0, s, p.partials, blocks, a->sums, a->flags);
+  hipLaunchKernelGGL(policy_loss_finalize_kernel, dim3(1), dim3(kNumSums * 64), 0, s, p.partials, blocks, a->sums, a->flags);
   return check_launch("policy_loss_finalize_kernel");
 }
 
