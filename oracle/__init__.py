@@ -14,7 +14,7 @@ of them, so none is pinned by a reference fixture):
   (uniform logits, one dominant logit, shift invariance, zero-sum gradient),
   a pure-Python row loop on tiny shapes, and torch's library routines.
 * GRPO / GSPO surrogate losses: closed forms for every clip branch
-  (``tests/test_oracle_losses.py``) and torch autograd for the tie gradients.
+  (``tests/test_oracle_cpu.py``) and torch autograd for the tie gradients.
 * k3 KL estimator: ``kl >= 0``, zero iff equal, derivative ``1 - exp(ref-lp)``.
 * bin packing: hand-worked cases stored in ``tests/golden/packing_cases.json``
   that exercise the strict-fit rule, first-on-ties and stable descending
@@ -28,6 +28,11 @@ of them, so none is pinned by a reference fixture):
   ``tests/golden/thd_pack_cases.json``; the context-parallel index split it
   calls from TransformerEngine is restated from the published chunk scheme and
   is PARITY UNPINNED for more than one rank (identity for one rank).
+* the FSDP trainer's micro-batch loops (``policy_loop.py``: preprocess_data_list, train_step,
+  forward_step): a three-sample case worked by hand from the reference lines with literal expected
+  tables (``tests/test_policy_loop_cpu.py``): micro-batch order with a tie on the bin totals, packed
+  row, indices, position ids, labels rolling across sequence boundaries, shifted training mask,
+  record lengths and values, train_stats and a row of the parameter gradient.
 * vocabulary-parallel logprob / entropy (the reference's three all-reduces
   over tensor-parallel ranks): equality with the unsharded log_softmax gather
   and entropy for every way of cutting the vocabulary, and the uniform-logits
