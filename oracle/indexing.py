@@ -80,14 +80,18 @@ def thd_partitioned_indices(cu_seqlens, total_tokens, world_size, rank):
     """Positions of a packed (THD) row that one context-parallel rank keeps.
 
     The reference calls TransformerEngine's ``tex.thd_get_partitioned_indices``
-    (megatron_utils/train_helper.py:289-291); TransformerEngine is a third-party
-    dependency that is not vendored, so this restates its published scheme: every
+    (megatron_utils/train_helper.py:289-291); TransformerEngine (2.7 in the reference's
+    images, docs/en/installation.md:28) is a third-party dependency that is not
+    vendored, so this restates its published scheme: every
     sequence is cut into ``2 * world_size`` equal chunks and rank ``r`` keeps chunks
     ``r`` and ``2 * world_size - 1 - r`` (load balancing under a causal mask), in
     sequence order.  For ``world_size == 1`` this is ``arange(total_tokens)``, which
     is all the reference's own single-rank use needs; for more ranks the parity of
     this function with TransformerEngine is unpinned (no fixture of it exists in the
-    reference) and only its defining properties are tested.
+    reference) and only its defining properties are tested
+    (tests/test_oracle_cpu.py::test_context_parallel_partition_properties): the ranks'
+    index sets partition the row, each is ascending, and every rank gets the same
+    amount of causal-attention work per sequence.
     """
     out = []
     for i in range(len(cu_seqlens) - 1):

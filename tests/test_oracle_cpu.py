@@ -332,3 +332,32 @@ def test_megatron_packed_batch_oracle_against_hand_worked_cases():
         assert out["labels"][0].tolist() == c["labels"]
         assert out["loss_mask_on_this_cp_rank"][:, 0].tolist() == c["loss_mask"]
         assert int(out["num_tokens_on_this_cp_rank"]) == c["num_tokens"] and int(out["pad_size"]) == c["pad_size"]
+
+
+@pytest.mark.parametrize("cp", [2, 4])
+def test_context_parallel_partition_properties(cp):
+    """What fixes the load-balanced split of a packed row over context-parallel ranks, without the
+    library the reference calls for it: the ranks' index sets partition the row, each is ascending
+    (sequence order is kept), each rank gets 1/cp of every sequence, and under a causal mask every
+    rank does the same amount of attention work per sequence (rank r pairs chunk r with chunk
+    2cp-1-r).  A literal case worked by hand closes the chunk numbering."""
+    lens = [4 * cp, 8 * cp, 2 * cp]
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    total = cu[-1]
+    parts = [oidx.thd_partitioned_indices(cu, total, cp, r) for r in range(cp)]
+    assert sorted(torch.cat(parts).tolist()) == list(range(total))
+    for part in parts:
+        assert part.tolist() == sorted(part.tolist()) and len(part) == total // cp
+    for s in range(len(lens)):
+        work = []
+        for part in parts:
+            mine = [int(i) - cu[s] for i in part.tolist() if cu[s] <= i < cu[s + 1]]
+            assert len(mine) == lens[s] // cp
+            work.append(sum(pos + 1 for pos in mine))     # keys a causal query at `pos` attends to
+        assert len(set(work)) == 1
+    if cp == 2:
+        # one sequence of 8 tokens, 4 chunks of 2: rank 0 keeps chunks 0 and 3, rank 1 chunks 1 and 2
+        assert oidx.thd_partitioned_indices([0, 8], 8, 2, 0).tolist() == [0, 1, 6, 7]
+        assert oidx.thd_partitioned_indices([0, 8], 8, 2, 1).tolist() == [2, 3, 4, 5]
