@@ -29,7 +29,7 @@ sys.path.insert(0, ROOT)
 
 from chatlearn_amd import _lib, ops, synthetic  # noqa: E402
 from chatlearn_amd._lib import LOSS_GRPO, LOSS_GSPO  # noqa: E402
-from chatlearn_amd.fused import DEFAULT_KEEP_LOGITS_TOKENS, _token_chunks, grpo_head_step  # noqa: E402
+from chatlearn_amd.fused import DEFAULT_KEEP_LOGITS_TOKENS, grpo_head_step, head_step_chunks  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3
@@ -112,7 +112,7 @@ def advantages_for(samples, device, group=1 << 30):
 
 
 def head_step(w, keep, dweight, *, skip_masked=True, skip_masked_forward=False, hook=None, accumulate=False,
-              weight_t_cache=None, n_tok=None):
+              weight_t_cache=None, n_tok=None, workspace_cache=None):
     cfg = w.cfg
     return grpo_head_step(w.hidden, w.weight, w.labels, w.old, w.ref, w.adv, w.cu, w.mask,
                           n_tokens_total=n_tok or w.n_tok, use_group_sequence_policy=(cfg.loss == "gspo"),
@@ -121,7 +121,8 @@ def head_step(w, keep, dweight, *, skip_masked=True, skip_masked_forward=False, 
                           entropy_coef=cfg.entropy_coef, temperature=cfg.temperature, dweight=dweight,
                           accumulate_dweight=accumulate, keep_logits_chunk=keep, cu_seqlens_host=w.cu_host,
                           skip_masked_rows=skip_masked, skip_masked_forward=skip_masked_forward, stage_hook=hook,
-                          loss_mask_host=w.mask_host, weight_t_cache=weight_t_cache, check_flags=False)
+                          loss_mask_host=w.mask_host, weight_t_cache=weight_t_cache, check_flags=False,
+                          workspace_cache=workspace_cache)
 
 
 def time_step(w, keep, dweight, steps, warmup, **kw):
@@ -130,6 +131,7 @@ def time_step(w, keep, dweight, steps, warmup, **kw):
     accumulated).  The no-grad configuration: fused forward only."""
     cfg = w.cfg
     marks = []
+    ws_cache = {}     # kept logits and scratch memory stay allocated between the steps, as a trainer's loop keeps them
 
     def once(record):
         if cfg.loss is None:
@@ -146,7 +148,7 @@ def time_step(w, keep, dweight, steps, warmup, **kw):
             ev = torch.cuda.Event(enable_timing=True)
             ev.record()
             cur.append((name, ev))
-        out = head_step(w, keep, dweight, hook=hook if record else None, **kw)
+        out = head_step(w, keep, dweight, hook=hook if record else None, workspace_cache=ws_cache, **kw)
         if record:
             marks.append(cur)
         return out
@@ -176,7 +178,7 @@ def step_record(w, keep, dt, stages, out):
     cfg = w.cfg
     train = cfg.loss is not None
     T = w.T
-    chunks = _token_chunks(T, keep, w.cu_host if (keep and cfg.loss == "gspo") else None) if train else [(0, T)]
+    chunks = out["token_chunks"] if train else [(0, T)]
     rows_fwd = out["rows_projected_fwd"] if train else T
     rows_bwd = out["rows_projected_bwd"] if train else 0
     hv = float(cfg.H) * cfg.V
@@ -324,7 +326,7 @@ def gemm_kernels(w, keep, reps=3):
     whole backward of the chunk and the backward without that output (what remains in either is the
     d(logits) pass and a transpose)."""
     cfg = w.cfg
-    chunks = _token_chunks(w.T, keep, w.cu_host if cfg.loss == "gspo" else None)
+    chunks = head_step_chunks(w.T, keep, cfg.loss == "gspo", w.cu_host, w.mask_host)
     lo, hi = max(chunks, key=lambda c: c[1] - c[0])
     n = hi - lo
     dev = w.device
@@ -541,18 +543,23 @@ def sweep(cfg, device, weight, keep):
         w.adv = adv_all[torch.tensor([s["sample_index"] for s in mb], device=device)]
         works.append(w.finish())
     dweight = torch.zeros(cfg.V, cfg.H, dtype=torch.float32, device=device)
-    cache = {}
+    cache, ws_cache = {}, {}
     for w in works[:2]:                                    # warm-up
-        head_step(w, keep, dweight, accumulate=True, weight_t_cache=cache, n_tok=n_tok_total)
+        head_step(w, keep, dweight, accumulate=True, weight_t_cache=cache, n_tok=n_tok_total, workspace_cache=ws_cache)
     cache.clear()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    rows_bwd = launches = 0
     for i, w in enumerate(works):
-        head_step(w, keep, dweight, accumulate=i > 0, weight_t_cache=cache, n_tok=n_tok_total)
+        o = head_step(w, keep, dweight, accumulate=i > 0, weight_t_cache=cache, n_tok=n_tok_total, workspace_cache=ws_cache)
+        rows_bwd += o["rows_projected_bwd"]
+        launches += len(o["token_chunks"])
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     tokens = sum(w.T for w in works)
-    return {"micro_batches": len(works), "tokens": tokens,
+    hv = float(cfg.H) * cfg.V
+    return {"micro_batches": len(works), "tokens": tokens, "T_projected_backward": rows_bwd, "token_chunks_total": launches,
+            "step_mfma_frac_executed": 2.0 * hv * (tokens + 2.0 * rows_bwd) / dt / 1e12 / peak_of(cfg),
             "tokens_per_micro_batch_min_max": [min(w.T for w in works), max(w.T for w in works)],
             "ms_total": dt * 1e3, "tokens_per_s": tokens / dt, "host_bin_packing_ms": round(packing_ms, 2),
             "note": "bin-packed micro-batches of the whole mini-batch, dW accumulated, W^T built once"}

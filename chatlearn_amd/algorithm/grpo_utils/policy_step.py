@@ -144,6 +144,7 @@ class PolicyStep:
         dw = self.dweight_buffer
         accumulate = dw is not None
         wt_cache = {}   # the weight does not change between the micro-batches of this step
+        ws_cache = {}   # kept logits and head scratch memory, shared by the micro-batches of this step
         for inputs in data_list:
             inputs = self._to_device(inputs)
             hidden = self.backbone(inputs["all_tokens"], inputs["position_ids"])
@@ -159,7 +160,8 @@ class PolicyStep:
                 accumulate_dweight=accumulate, need_dhidden=flat.requires_grad,
                 keep_logits_chunk=self.keep_logits_chunk,
                 # only masked sums leave this method, so rows outside the loss mask need no forward either
-                skip_masked_forward=True, weight_t_cache=wt_cache, loss_mask_host=inputs["loss_mask_host"])
+                skip_masked_forward=True, weight_t_cache=wt_cache, loss_mask_host=inputs["loss_mask_host"],
+                workspace_cache=ws_cache)
             dw, accumulate = out["dweight"], True
             if flat.requires_grad:
                 hidden.backward(out["dhidden"].reshape(hidden.shape))

@@ -12,6 +12,7 @@ loss (+ upstream gradients), fused backward - for callers that own the training
 loop; it walks the micro-batch in token chunks and lets the backward reuse the
 chunk's logits instead of recomputing them.
 """
+import bisect
 from typing import Optional
 
 import torch
@@ -191,35 +192,83 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     return lp, ent
 
 
-def _token_chunks(T, chunk_tokens, seq_bounds):
-    """[lo, hi) token ranges of at most ``chunk_tokens`` tokens, as few as that allows and of about
-    equal size (a small last range would run the backward GEMMs at poor efficiency).  With
-    ``seq_bounds`` (the host copy of cu_seqlens) every range ends on a sequence boundary; a range
-    exceeds ``chunk_tokens`` only where a single sequence is longer than it."""
-    if chunk_tokens is None or chunk_tokens >= T:
+def _token_chunks(T, chunk_rows, seq_bounds, live_cum=None):
+    """[lo, hi) token ranges holding at most ``chunk_rows`` rows each: as few ranges as that allows, and
+    of about equal length in tokens (the forward runs on every token of a range; a short last range would
+    run all kernels at poor efficiency).  A token counts as a row, unless ``live_cum`` is given (a numpy
+    array, live_cum[i] = rows among tokens [0, i) whose logits are kept, i.e. the unmasked ones): then the
+    bound is on those.  With ``seq_bounds`` (the host copy of cu_seqlens) every range ends on a sequence
+    boundary (a range exceeds ``chunk_rows`` only where a single sequence is larger than it), otherwise
+    on a multiple of 256 tokens where the bound leaves room for that."""
+    total = T if live_cum is None else int(live_cum[T])
+    if chunk_rows is None or chunk_rows >= total or T == 0:
         return [(0, T)]
-    cuts = sorted(set(int(x) for x in seq_bounds if 0 < int(x) < T)) + [T] if seq_bounds is not None else None
-    # number of ranges a greedy fill needs: the balanced cut below aims at that many
+    wt = (lambda pos: pos) if live_cum is None else (lambda pos: int(live_cum[pos]))
+
+    def first_with(rows):       # smallest position with at least `rows` rows before it
+        return min(T, rows) if live_cum is None else min(T, int(live_cum.searchsorted(rows, side="left")))
+
+    def last_with(rows):        # largest position with at most `rows` rows before it
+        return min(T, rows) if live_cum is None else min(T, int(live_cum.searchsorted(rows, side="right")) - 1)
+
+    cuts = wcuts = None
+    if seq_bounds is not None:
+        cuts = sorted(set(int(x) for x in seq_bounds if 0 < int(x) < T)) + [T]
+        wcuts = [wt(c) for c in cuts]
+
+    def choose(lo, need, target):
+        """End of the range that starts at lo: within the bound, leaving at most `total - need` rows behind
+        where possible, and as near to token `target` as those two allow."""
+        limit = wt(lo) + chunk_rows
+        if cuts is None:
+            hi_max = max(lo + 1, last_with(limit))
+            hi_min = min(hi_max, max(lo + 1, first_with(need)))
+            hi = min(max(target, hi_min), hi_max)
+            for r in sorted({hi // 256 * 256, (hi + 255) // 256 * 256}, key=lambda r: abs(r - hi)):
+                if hi_min <= r <= hi_max and r < T:
+                    return r
+            return hi
+        a = bisect.bisect_right(cuts, lo)
+        b = max(a + 1, bisect.bisect_right(wcuts, limit))          # a single longer sequence gets a range of its own
+        a2 = min(max(bisect.bisect_left(wcuts, need, a, b), a), b - 1)
+        return min(cuts[a2:b], key=lambda c: (abs(c - target), c))
+
+    # number of ranges: fill each to the bound
     n, lo = 0, 0
     while lo < T:
-        if cuts is None:
-            lo = min(T, lo + chunk_tokens)
-        else:
-            ok = [c for c in cuts if lo < c <= lo + chunk_tokens]
-            lo = max(ok) if ok else min(c for c in cuts if c > lo)
+        lo = choose(lo, total, T)
+        if wt(lo) == total:
+            lo = T                                                 # a tail without rows rides along
         n += 1
     out, lo = [], 0
     while lo < T:
-        left = max(-(-(T - lo) // chunk_tokens), n - len(out), 1)
-        target = lo + -(-(T - lo) // left)
-        if cuts is None:
-            hi = min(T, target)
+        left = n - len(out)
+        if left <= 1 and total - wt(lo) <= chunk_rows:
+            hi = T
         else:
-            ok = [c for c in cuts if lo < c <= lo + chunk_tokens]
-            hi = min(ok, key=lambda c: (abs(c - target), c)) if ok else min(c for c in cuts if c > lo)
+            left = max(left, 2)
+            hi = choose(lo, total - (left - 1) * chunk_rows, lo + -(-(T - lo) // left))
+            if wt(hi) == total:
+                hi = T
         out.append((lo, hi))
         lo = hi
     return out
+
+
+def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask_host=None):
+    """The token ranges ``grpo_head_step`` walks: at most ``keep_logits_chunk`` kept rows each.  Only
+    unmasked rows keep their logits, so with the mask known on the host (``loss_mask_host``, given when
+    masked rows are skipped) the bound counts those; the sequence-level loss needs ranges that end on
+    sequence boundaries (``cu_seqlens``: host list or device tensor, read only when a split is needed)."""
+    live_cum = None
+    if loss_mask_host is not None and T > 0:
+        live_cum = torch.cat([torch.zeros(1, dtype=torch.int64),
+                              (loss_mask_host.reshape(-1) != 0).to(torch.int64).cumsum(0)]).numpy()
+    rows_total = T if live_cum is None else int(live_cum[T])
+    bounds = None
+    if keep_logits_chunk is not None and keep_logits_chunk < rows_total and sequence_level:
+        bounds = cu_seqlens.tolist() if isinstance(cu_seqlens, torch.Tensor) else list(cu_seqlens)
+    return _token_chunks(T, keep_logits_chunk, bounds, live_cum)
 
 
 def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages, cu_seqlens, loss_mask, *,
@@ -229,7 +278,8 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                    accumulate_dweight=False, need_dhidden=True, check_flags=True,
                    keep_logits_chunk: Optional[int] = DEFAULT_KEEP_LOGITS_TOKENS, cu_seqlens_host=None,
                    skip_masked_rows=True, skip_masked_forward=False, weight_t_cache: Optional[dict] = None,
-                   stage_hook=None, loss_mask_host: Optional[torch.Tensor] = None):
+                   stage_hook=None, loss_mask_host: Optional[torch.Tensor] = None,
+                   workspace_cache: Optional[dict] = None):
     """Forward + loss + backward of the head for one packed micro-batch, no autograd graph.
 
     Mirrors policy_trainer.py:216-286 on packed rows: returns a dict with the
@@ -237,9 +287,10 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     ``kl_loss_mean``, ``entropy_loss_mean``, ``total_loss`` (device fp64 scalars),
     ``dhidden`` and ``dweight``.  ``advantages`` is a device tensor [B].
 
-    ``keep_logits_chunk``: the micro-batch is walked in chunks of about this many tokens; within
-    a chunk the forward keeps its raw logits (one [chunk, V] buffer in the input dtype, reused
-    chunk after chunk) so the backward does not recompute them.  ``None`` keeps nothing: the
+    ``keep_logits_chunk``: the micro-batch is walked in token chunks that keep the raw logits of at most
+    this many rows (one [chunk, V] buffer of 16-bit or fp32 elements, reused chunk after chunk) so that
+    the backward does not recompute them.  Every token counts as a row, except that with
+    ``skip_masked_rows`` and ``loss_mask_host`` only the unmasked tokens do (only they are kept).  ``None`` keeps nothing: the
     backward then recomputes the logit tiles from ``hidden`` and ``weight``.  The sequence-level
     loss needs chunks that end on sequence boundaries, so it reads ``cu_seqlens_host`` (or copies
     ``cu_seqlens`` to the host once).
@@ -262,6 +313,12 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     of one optimizer step).  The first backward leaves the transposed weight in it and later calls
     reuse it instead of transposing again; the caller clears it after updating the weight.
 
+    ``workspace_cache``: a dict the caller keeps between calls.  The kept-logits buffer and the forward /
+    backward scratch memory (a few GB, sized by the chunk, not by T) then live in it and are reused by every
+    later call they are large enough for, instead of being allocated and released per call: micro-batches of
+    varying length otherwise ask the framework's allocator for differently sized multi-GB blocks each time,
+    which now and then costs a device-wide stall for a fresh allocation.
+
     ``stage_hook(name)`` is called on the host at "forward", "loss", "backward", "end" boundaries
     of every chunk (a benchmark records stream events there).
     """
@@ -270,23 +327,32 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     V = weight.shape[0]
     scale = float(fsdp_size) / float(n_tokens_total)
     mode = LOSS_GSPO if use_group_sequence_policy else LOSS_GRPO
-    bounds = None
-    if keep_logits_chunk is not None and keep_logits_chunk < T and use_group_sequence_policy:
-        bounds = list(cu_seqlens_host) if cu_seqlens_host is not None else cu_seqlens.tolist()
-    chunks = _token_chunks(T, keep_logits_chunk, bounds)
-    zbuf = None
     skip = keep_logits_chunk is not None and loss_mask is not None and skip_masked_rows
+    chunks = head_step_chunks(T, keep_logits_chunk, use_group_sequence_policy,
+                              cu_seqlens_host if cu_seqlens_host is not None else cu_seqlens,
+                              loss_mask_host if skip else None)
+    zbuf = None
     rows_of = None
     if skip and loss_mask_host is not None and T > 0:
         rows_of = _live_rows_from_host_mask(loss_mask_host, chunks, hidden.device)
     longest = max(hi - lo for lo, hi in chunks)
+    cache = workspace_cache if workspace_cache is not None else {}
+
+    def scratch(name, nbytes):
+        buf = cache.get(name)
+        if buf is None or buf.numel() < nbytes or buf.device != hidden.device:
+            buf = cache[name] = torch.empty(nbytes, dtype=torch.uint8, device=hidden.device)
+        return buf
+
     if keep_logits_chunk is not None and T > 0:
         kept = longest if rows_of is None else max(int(live.numel()) for live, _ in rows_of)
-        zbuf = ops.saved_logits_buffer(kept, V, hidden.dtype, hidden.device)
+        zbuf = cache.get("kept_logits")
+        if zbuf is None or zbuf.shape[0] < kept or zbuf.dtype != hidden.dtype or zbuf.device != hidden.device \
+                or zbuf.shape[1] != ops.saved_logits_ld(V):
+            zbuf = cache["kept_logits"] = ops.saved_logits_buffer(kept, V, hidden.dtype, hidden.device)
     # scratch memory of the forward and the backward, shared by all chunks of this call
     H = hidden.shape[1]
-    fwd_ws = torch.empty(max(ops.lmhead_forward_workspace_bytes(longest, H, V, hidden.dtype), 16), dtype=torch.uint8,
-                         device=hidden.device) if T > 0 else None
+    fwd_ws = scratch("forward", max(ops.lmhead_forward_workspace_bytes(longest, H, V, hidden.dtype), 16)) if T > 0 else None
     bwd_rows = longest if zbuf is None else min(longest, zbuf.shape[0])
     bwd_ws = None
     f = dict(dtype=torch.float32, device=hidden.device)
@@ -306,8 +372,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     if need_dhidden and wt is None and (len(chunks) > 1 or weight_t_cache is not None):
         wt = ops.weight_t_buffer(weight)
     if zbuf is not None:
-        bwd_ws = torch.empty(ops.lmhead_backward_workspace_bytes(bwd_rows, H, V, hidden.dtype, True, wt is not None),
-                             dtype=torch.uint8, device=hidden.device)
+        bwd_ws = scratch("backward", ops.lmhead_backward_workspace_bytes(bwd_rows, H, V, hidden.dtype, True, wt is not None))
     kl_c = kl_coef if kl_coef > 0 else 0.0
     en_c = entropy_coef if entropy_coef > 0 else 0.0
     for k, (lo, hi) in enumerate(chunks):
@@ -399,7 +464,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
             "entropy_loss_mean": en, "total_loss": total, "num_masked": sums[3],
             "per_token_loss": loss_all, "per_token_kl": kl_all, "dhidden": dh_all, "dweight": dw,
             "g_logprob": glp_all, "rows_projected_bwd": rows_projected_bwd,
-            "rows_projected_fwd": rows_projected_fwd, "sums": sums,
+            "rows_projected_fwd": rows_projected_fwd, "sums": sums, "token_chunks": chunks,
             # device memory this call held beyond its inputs and outputs: kept logits (they become d(logits) in
             # place), the backward's operands (d(logits)^T, hidden^T, W^T unless the caller's cache holds it,
             # split-K partials) and the forward's per-split records

@@ -49,6 +49,11 @@ def _round_up(x: int, m: int) -> int:
     return (x + m - 1) // m * m
 
 
+def saved_logits_ld(V: int) -> int:
+    """Elements per row of a kept-logits buffer for a vocabulary of V entries."""
+    return int(_lib.lib().clgrpo_saved_logits_ld(V))
+
+
 def saved_logits_buffer(T: int, V: int, dtype, device) -> torch.Tensor:
     """An (uninitialised) buffer the forward can keep raw logits in for the backward: T rows rounded
     up to whole blocks of 256 by the padded vocabulary extent, elements of the size of ``dtype``.  Its
@@ -583,7 +588,7 @@ def thd_pack(tokens: torch.Tensor, prompt_len, response_len, align: int, pad_tok
                          _ptr(cu), _ptr(seqlens), _ptr(seqlens_padded), _ptr(stats), _ptr(status), _ptr(indices),
                          _ptr(seq_indices), _ptr(out_tokens), _ptr(out_labels), _ptr(out_mask), _ptr(out_pos))
     _lib.call("clgrpo_thd_pack", a, _stream(tokens))
-    # the device recomputes the sizes from the same lengths; reading its verdict costs a host round trip
+    # the device recomputes the sizes from the same lengths; reading its result back costs a host round trip
     bad = int(status.item()) if verify_on_device else 0
     if bad:
         why = [m for bit, m in ((1, "padded total differs from the host's"), (2, "a sequence is longer than S"),

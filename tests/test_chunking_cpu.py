@@ -1,13 +1,15 @@
 """Token chunking of a micro-batch (host logic of grpo_head_step)."""
 import random
 
+import numpy as np
+
 from chatlearn_amd.fused import _token_chunks
 
 
 def test_hand_worked_chunks():
     assert _token_chunks(16384, 16384, None) == [(0, 16384)]
     assert _token_chunks(16384, None, None) == [(0, 16384)]
-    assert _token_chunks(20000, 16384, None) == [(0, 10000), (10000, 20000)]              # two equal ranges, not 16384 + 3616
+    assert _token_chunks(20000, 16384, None) == [(0, 9984), (9984, 20000)]                # two about equal ranges cut on a multiple of 256, not 16384 + 3616
     assert _token_chunks(100, 30, None) == [(0, 25), (25, 50), (50, 75), (75, 100)]
     bounds = [0, 4000, 9000, 11000, 15169, 20000, 22000, 29588, 32768]
     assert _token_chunks(32768, 16384, bounds) == [(0, 11000), (11000, 22000), (22000, 32768)]
@@ -32,3 +34,37 @@ def test_chunk_properties_on_random_layouts():
             for lo, hi in ranges:
                 if hi - lo > cap:
                     assert not any(lo < x < hi for x in bounds)                            # a single long sequence
+
+
+def test_chunks_bounded_by_kept_rows():
+    """With the unmasked rows counted (only they keep logits) the bound is on those: fewer, longer token
+    ranges; tokens or sequences without a kept row never open a range of their own."""
+    live = np.array([1, 1, 0, 0, 1, 0, 1, 1, 0, 0, 0, 0])
+    cum = np.concatenate([[0], np.cumsum(live)])
+    assert _token_chunks(12, 3, None, cum) == [(0, 6), (6, 12)]                            # 3 + 2 kept rows, the masked tail rides along
+    assert _token_chunks(12, 5, None, cum) == [(0, 12)]
+    assert _token_chunks(12, 2, [0, 2, 4, 8, 12], cum) == [(0, 4), (4, 12)]                # sequence [2, 4) has no kept row
+    rng = random.Random(2)
+    for _ in range(2000):
+        T = rng.randint(1, 4000)
+        keep_p = rng.choice([0.05, 0.5, 0.75, 1.0])
+        live = np.array([1 if rng.random() < keep_p else 0 for _ in range(T)])
+        if rng.random() < 0.3:
+            live[rng.randint(0, T - 1):] = 0                                               # masked tail
+        cum = np.concatenate([[0], np.cumsum(live)])
+        cap = rng.randint(1, 2500)
+        bounds = sorted({0, T} | {rng.randint(1, T) for _ in range(rng.randint(1, 30))}) if rng.random() < 0.5 else None
+        ranges = _token_chunks(T, cap, bounds, cum)
+        assert ranges[0][0] == 0 and ranges[-1][1] == T
+        assert all(a[1] == b[0] for a, b in zip(ranges, ranges[1:])) and all(hi > lo for lo, hi in ranges)
+        rows = [int(cum[hi] - cum[lo]) for lo, hi in ranges]
+        if bounds is None:
+            assert all(r <= cap for r in rows)
+            assert len(ranges) == max(1, -(-int(cum[T]) // cap))                           # as few as the cap allows
+        else:
+            assert all(hi in bounds for _, hi in ranges)
+            for (lo, hi), r in zip(ranges, rows):
+                if r > cap:
+                    assert not any(lo < x < hi and cum[lo] < cum[x] < cum[hi] for x in bounds)
+        if len(ranges) > 1:
+            assert rows[-1] > 0 or bounds is not None                                      # no range for a tail without kept rows
