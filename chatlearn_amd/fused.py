@@ -92,19 +92,22 @@ def _live_rows_from_host_mask(mask_host: torch.Tensor, chunks, device):
 
 class _FusedHead(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, labels, temperature, need_entropy, dweight_buffer, keep_logits, row_mask):
+    def forward(ctx, hidden, weight, labels, temperature, need_entropy, dweight_buffer, keep_rows, row_mask):
         T = hidden.shape[0]
         zbuf = live = row_map = None
-        if keep_logits and T > 0:
+        if keep_rows is not None and T > 0:
             if row_mask is not None:
                 # rows outside the mask get a zero upstream gradient whatever their logits are:
                 # keep logits only for the others and run the backward on that compact set
                 live = _nonzero_rows(row_mask)
-                row_map = torch.full((T,), -1, dtype=torch.int32, device=hidden.device)
-                row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
             rows = T if live is None else int(live.numel())
-            if rows > 0:
+            if rows > keep_rows:
+                live = None                  # more rows than may be kept: the backward recomputes its logit tiles
+            elif rows > 0:
                 zbuf = ops.saved_logits_buffer(rows, weight.shape[0], hidden.dtype, hidden.device)
+                if live is not None:
+                    row_map = torch.full((T,), -1, dtype=torch.int32, device=hidden.device)
+                    row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
         lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, temperature, need_entropy,
                                              saved_logits=zbuf, saved_row_map=row_map if zbuf is not None else None)
         ctx.save_for_backward(hidden, weight, labels, lse, ent if ent is not None else lse)
@@ -167,8 +170,8 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     without it ``weight.grad`` gets dW cast to the weight dtype, as torch would.
     Leading dimensions of hidden/labels are flattened and restored.
 
-    ``keep_logits_rows``: when a gradient is needed and there are at most this many rows, the forward
-    keeps its raw logits (one 16-bit copy for 16-bit inputs, released by the backward) so that the
+    ``keep_logits_rows``: when a gradient is needed and there are at most this many rows (with
+    ``loss_mask``: unmasked rows), the forward keeps their raw logits (one 16-bit copy for 16-bit inputs, released by the backward) so that the
     backward does not recompute them; ``None`` or more rows: recompute.  The default bounds the kept
     logits at 2.5 GB for a 152k vocabulary; a caller that wants the fast path for a larger micro-batch
     either raises it or runs the head chunk by chunk (forward, loss, backward per chunk), which is what
@@ -181,9 +184,9 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     h2 = hidden.reshape(-1, hidden.shape[-1])
     T = h2.shape[0]
     needs_grad = torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad)
-    keep = bool(needs_grad and keep_logits_rows is not None and T <= keep_logits_rows)
+    keep = keep_logits_rows if needs_grad else None      # rows whose logits may be kept; None: keep nothing
     mask = None
-    if keep and loss_mask is not None:
+    if keep is not None and loss_mask is not None:
         mask = loss_mask.reshape(-1).to(torch.int32)
     lp, ent = _FusedHead.apply(h2, weight, labels.reshape(-1), float(temperature), bool(need_entropy), dweight_buffer,
                                keep, mask)
