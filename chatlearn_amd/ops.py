@@ -12,7 +12,10 @@ import torch
 from . import _lib
 from ._lib import BF16, F32, F64, U8, LOSS_GRPO, LOSS_GSPO
 
-DEFAULT_BWD_WORKSPACE_BYTES = 24 << 30
+# Scratch memory a backward call may take when the caller names neither a chunk nor a workspace: the
+# token chunk is halved until the plan fits (8192 tokens of a 152k vocabulary need 6.5 GB: d(logits) in
+# both orientations, hidden^T, W^T, split-K partials).
+DEFAULT_BWD_WORKSPACE_BYTES = 8 << 30
 
 
 def _dtype_enum(t: torch.Tensor) -> int:
