@@ -214,3 +214,40 @@ def test_backward_weight_gradient_with_walking_workgroups(dev):
     ops.lmhead_backward(hd, wd, ld, lse, ent, g_lp.to(dev), g_ent.to(dev), 1.0, need_dhidden=False, dweight=acc,
                         accumulate_dweight=True)
     assert_close_rel(acc - base.to(dev), rdw, 1e-2, "accumulated dweight")
+
+
+EDGE_SHAPES = [
+    # T, H, V, dtype: tile edges in every dimension (tokens around 256, vocabulary around 32 / 64 / 256, the smallest H)
+    (2, 64, 33, torch.bfloat16), (255, 64, 63, torch.bfloat16), (257, 128, 64, torch.bfloat16),
+    (511, 64, 65, torch.bfloat16), (64, 192, 255, torch.bfloat16), (769, 64, 513, torch.bfloat16),
+    (3, 32, 31, torch.float32), (256, 32, 256, torch.float32), (258, 96, 289, torch.float32),
+]
+
+
+@pytest.mark.parametrize("T,H,V,dtype", EDGE_SHAPES)
+def test_edge_shapes_forward_and_both_backward_routes(dev, T, H, V, dtype):
+    """Shapes that end inside a tile in every dimension: forward against the oracle, then the backward twice -
+    recomputing the logit tiles, and from logits the forward kept - against the oracle's closed form."""
+    from chatlearn_amd import ops
+    hidden, weight, labels = _inputs(T, H, V, dtype, seed=7 * T + V, w_std=0.2)
+    g = torch.Generator().manual_seed(T)
+    g_lp, g_ent = torch.randn(T, generator=g), torch.randn(T, generator=g) * 0.1
+    g_lp[::3] = 0.0
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    r = RTOL[dtype]
+    rlp, rent, _, rlse = osm.fused_head_forward(hidden, weight, labels, 1.0, torch.float64)
+    rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, g_lp, g_ent, 1.0)
+    zbuf = ops.saved_logits_buffer(T, V, dtype, dev)
+    for saved in (None, zbuf):
+        lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld, 1.0, need_entropy=True, saved_logits=saved)
+        assert_close_rel(lp, rlp, r, "logprob")
+        assert_close_rel(ent, rent, r, "entropy")
+        assert_close_rel(lse, rlse, r, "lse")
+        if saved is not None:
+            z = ops.saved_logits_rowmajor(saved, T, V).double().cpu()
+            assert_close_rel(z, hidden.double() @ weight.double().t(), 2 ** -10 if dtype != torch.float32 else 1e-5, "kept logits")
+        dh, dw = ops.lmhead_backward(hd, wd, ld, lse, ent, g_lp.to(dev), g_ent.to(dev), 1.0, saved_logits=saved)
+        route = "kept logits" if saved is not None else "recompute"
+        assert_close_rel(dh, rdh, r, f"dhidden ({route})")
+        assert_close_rel(dw, rdw, r, f"dweight ({route})")
+        assert torch.isfinite(dh.float()).all() and torch.isfinite(dw).all()
