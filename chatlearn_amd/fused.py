@@ -15,6 +15,7 @@ chunk's logits instead of recomputing them.
 import bisect
 from typing import Optional
 
+import numpy as np
 import torch
 
 from . import ops
@@ -73,20 +74,21 @@ def _upload(host: torch.Tensor, device) -> torch.Tensor:
 def _live_rows_from_host_mask(mask_host: torch.Tensor, chunks, device):
     """Per token chunk: (positions of the unmasked rows inside the chunk, int64; row map int32 with the
     rank of each unmasked row or -1), built on the host from a host copy of the loss mask and sent
-    over in two asynchronous copies, so that no device value has to be read back."""
-    flat = mask_host.reshape(-1) != 0
-    live_all = torch.nonzero(flat).flatten()
-    bounds = torch.searchsorted(live_all, torch.tensor([lo for lo, _ in chunks] + [chunks[-1][1]]))
-    local = live_all.clone()
-    row_map = torch.full((flat.numel(),), -1, dtype=torch.int32)
+    over in two asynchronous copies, so that no device value has to be read back.  The index work is
+    numpy's (single-threaded): a few microseconds, and no thread pool to wake on the step's critical path."""
+    flat = mask_host.reshape(-1).numpy() != 0
+    live_all = np.flatnonzero(flat).astype(np.int64)
+    bounds = np.searchsorted(live_all, [lo for lo, _ in chunks] + [chunks[-1][1]])
+    local = live_all.copy()
+    row_map = np.full(flat.shape[0], -1, dtype=np.int32)
     counts = []
     for k, (lo, hi) in enumerate(chunks):
         a, b = int(bounds[k]), int(bounds[k + 1])
         local[a:b] -= lo
-        row_map[live_all[a:b]] = torch.arange(b - a, dtype=torch.int32)
+        row_map[live_all[a:b]] = np.arange(b - a, dtype=np.int32)
         counts.append((a, b))
-    local_d = _upload(local, device) if local.numel() else torch.empty(0, dtype=torch.int64, device=device)
-    map_d = _upload(row_map, device)
+    local_d = _upload(torch.from_numpy(local), device) if local.size else torch.empty(0, dtype=torch.int64, device=device)
+    map_d = _upload(torch.from_numpy(row_map), device)
     return [(local_d[a:b], map_d[lo:hi]) for (a, b), (lo, hi) in zip(counts, chunks)]
 
 
@@ -265,8 +267,7 @@ def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask
     sequence boundaries (``cu_seqlens``: host list or device tensor, read only when a split is needed)."""
     live_cum = None
     if loss_mask_host is not None and T > 0:
-        live_cum = torch.cat([torch.zeros(1, dtype=torch.int64),
-                              (loss_mask_host.reshape(-1) != 0).to(torch.int64).cumsum(0)]).numpy()
+        live_cum = np.concatenate([[0], np.cumsum(loss_mask_host.reshape(-1).numpy() != 0, dtype=np.int64)])
     rows_total = T if live_cum is None else int(live_cum[T])
     bounds = None
     if keep_logits_chunk is not None and keep_logits_chunk < rows_total and sequence_level:
