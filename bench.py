@@ -419,6 +419,19 @@ def glue_stages(cfg, samples, device, reps=20):
                                     want_upstream=True), T * 44, _lib.lib().clgrpo_policy_loss_launches(T, 0)),
         "group advantages (whole episode, host grouping + kernel)": (advantages, len(pop) * 24, 1),
     }
+    # The statistics kernels for callers that already hold logits (the reference's logprobs_from_logits /
+    # entropy_from_logits mirrors): HBM-bound, so their GB/s is against the 8 TB/s peak.  2048 rows of the
+    # full vocabulary in the workload's dtype.
+    R = 2048
+    logits = torch.randn(R, cfg.V, generator=gen, device=device, dtype=torch.float32).to(cfg.dtype)
+    lab = torch.randint(0, cfg.V, (R,), generator=gen, device=device)
+    es = logits.element_size()
+    s_lp, s_ent, s_lse = ops.softmax_stats(logits, lab)
+    g1 = torch.randn(R, generator=gen, device=device)
+    stages["softmax_stats (logprob + entropy from logits) [2048,V]"] = (
+        lambda: ops.softmax_stats(logits, lab), R * cfg.V * es, 1)
+    stages["softmax_stats_backward (d logits, statistics from the forward) [2048,V]"] = (
+        lambda: ops.softmax_stats_backward(logits, lab, g1, g1, lse=s_lse, entropy=s_ent), 2 * R * cfg.V * es, 1)
     out = {}
     for name, (fn, nbytes, launches) in stages.items():
         for _ in range(3):

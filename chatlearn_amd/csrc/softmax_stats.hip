@@ -48,15 +48,17 @@ __device__ __forceinline__ void rs_update(RowStats& st, const float (&z)[N]) {
   float vmax = z[0];
 #pragma unroll
   for (int k = 1; k < N; ++k) vmax = fmaxf(vmax, z[k]);
+  constexpr float kLog2e = 1.4426950408889634f;
   if (vmax > st.m) {
-    const float f = expf(st.m - vmax);   // st.m = -inf -> 0
+    const float f = __builtin_amdgcn_exp2f((st.m - vmax) * kLog2e);   // st.m = -inf -> 0
     st.s *= f;
     st.u *= f;
     st.m = vmax;
   }
+  const float nb = -st.m * kLog2e;
 #pragma unroll
   for (int k = 0; k < N; ++k) {
-    const float e = expf(z[k] - st.m);
+    const float e = __builtin_amdgcn_exp2f(fmaf(z[k], kLog2e, nb));   // one hardware exp2 per element
     st.s += e;
     st.u = fmaf(e, z[k], st.u);
   }
@@ -78,14 +80,17 @@ __device__ RowStats row_stats(const T* row, int64_t V, bool vec) {
     const u32x4_t* rv = reinterpret_cast<const u32x4_t*>(row);
     const int64_t nvec = V / N;
     int64_t i = threadIdx.x;
+    // two independent running states per thread (merged below): the update is a dependent chain
+    RowStats st2{-INFINITY, 0.f, 0.f};
     for (; i + 3 * 256 < nvec; i += 4 * 256) {
       const u32x4_t r0 = rv[i], r1 = rv[i + 256], r2 = rv[i + 512], r3 = rv[i + 768];
-      float z[N];
-      Vec16<T>::unpack(r0, z); rs_update<N>(st, z);
-      Vec16<T>::unpack(r1, z); rs_update<N>(st, z);
-      Vec16<T>::unpack(r2, z); rs_update<N>(st, z);
-      Vec16<T>::unpack(r3, z); rs_update<N>(st, z);
+      float z[N], y[N];
+      Vec16<T>::unpack(r0, z); Vec16<T>::unpack(r1, y);
+      rs_update<N>(st, z); rs_update<N>(st2, y);
+      Vec16<T>::unpack(r2, z); Vec16<T>::unpack(r3, y);
+      rs_update<N>(st, z); rs_update<N>(st2, y);
     }
+    rs_merge(st, st2);
     for (; i < nvec; i += 256) {
       float z[N];
       Vec16<T>::unpack(rv[i], z);
@@ -151,7 +156,7 @@ __global__ __launch_bounds__(256) void softmax_stats_bwd_kernel(clgrpo_softmax_s
   const int64_t y = a.g_logprob ? a.labels[r] : -1;
   auto dz = [&](float z, int64_t v) {
     const float logp = z - lse;
-    const float p = expf(logp);
+    const float p = __builtin_amdgcn_exp2f(logp * 1.4426950408889634f);
     float d = -p * (glp + gen * (logp + ent));
     if (v == y) d += glp;
     return d;
