@@ -55,7 +55,7 @@ __device__ __forceinline__ void rs_update(RowStats& st, const float (&z)[N]) {
     st.u *= f;
     st.m = vmax;
   }
-  const float nb = -st.m * kLog2e;
+  const float nb = (st.m == -INFINITY) ? 0.f : -st.m * kLog2e;   // only -inf so far (masked entries): every term is 0
 #pragma unroll
   for (int k = 0; k < N; ++k) {
     const float e = __builtin_amdgcn_exp2f(fmaf(z[k], kLog2e, nb));   // one hardware exp2 per element

@@ -182,3 +182,25 @@ def test_stats_from_logits_mirrors(dev, dtype, V):
     d_with = ops.softmax_stats_backward(half, lab_h, gl, ge, lse=lse_h, entropy=en_h)
     d_without = ops.softmax_stats_backward(half, lab_h, gl, ge)
     assert_close_rel(d_with, d_without, 1e-5 if dtype == torch.float32 else 2 ** -7, "backward with / without kept statistics")
+
+
+def test_stats_from_logits_with_masked_vocabulary_entries(dev):
+    """Rows whose leading (or scattered) entries are -inf, as a vocabulary mask produces them: those entries
+    contribute nothing to lse and logprob (torch's logsumexp semantics).  The entropy of such a row is NaN in
+    the reference's formula (softmax * logits has 0 * -inf terms, trainer_utils.py:76-80) and NaN here."""
+    from chatlearn_amd import ops
+    g = torch.Generator().manual_seed(9)
+    R, V = 37, 4096
+    z = torch.randn(R, V, generator=g) * 3
+    z[:20, :2100] = float("-inf")                   # every thread's first pieces are all -inf
+    z[5, 3000:3500] = float("-inf")
+    labels = torch.randint(2100, 3000, (R,), generator=g)
+    lp, ent, lse = ops.softmax_stats(z.to(dev), labels.to(dev))
+    z64 = z.double()
+    want_lse = torch.logsumexp(z64, dim=-1)
+    want_ent = want_lse - (torch.softmax(z64, dim=-1) * z64).sum(-1)       # the reference's expression
+    assert torch.isfinite(lse).all()
+    assert_close_rel(lse, want_lse, 1e-5, "lse")
+    assert_close_rel(lp, z64.gather(1, labels[:, None])[:, 0] - want_lse, 1e-5, "logprob")
+    assert torch.equal(torch.isnan(ent).cpu(), torch.isnan(want_ent)) and int(torch.isnan(want_ent).sum()) == 20
+    assert_close_rel(ent[20:], want_ent[20:], 1e-5, "entropy of the unmasked rows")
