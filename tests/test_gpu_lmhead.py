@@ -251,3 +251,36 @@ def test_edge_shapes_forward_and_both_backward_routes(dev, T, H, V, dtype):
         assert_close_rel(dh, rdh, r, f"dhidden ({route})")
         assert_close_rel(dw, rdw, r, f"dweight ({route})")
         assert torch.isfinite(dh.float()).all() and torch.isfinite(dw).all()
+
+
+def test_backward_option_combinations_agree(dev):
+    """The backward's routes and options on one input: recompute or kept logits, one pass or token chunks,
+    the caller's W^T buffer (fresh, then marked ready), dW written or added to.  All must give the gradients
+    of the plain call (up to the fp32 summation order and, for kept logits, the half rounding of the logits)."""
+    from chatlearn_amd import ops
+    T, H, V = 1100, 192, 2500
+    hidden, weight, labels = _inputs(T, H, V, torch.bfloat16, seed=21, w_std=0.1)
+    g = torch.Generator().manual_seed(22)
+    g_lp, g_ent = torch.randn(T, generator=g), torch.randn(T, generator=g) * 0.1
+    g_lp[::4] = 0.0
+    hd, wd, ld, gl, ge = hidden.to(dev), weight.to(dev), labels.to(dev), g_lp.to(dev), g_ent.to(dev)
+    lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld)
+    dh0, dw0 = ops.lmhead_backward(hd, wd, ld, lse, ent, gl, ge)
+    wt = ops.weight_t_buffer(wd)
+    wt_ready = False
+    for saved in (False, True):
+        for chunk in (None, 256, 512):
+            for accumulate in (False, True):
+                zbuf = None
+                if saved:
+                    zbuf = ops.saved_logits_buffer(T, V, torch.bfloat16, dev)
+                    ops.lmhead_forward(hd, wd, ld, saved_logits=zbuf)
+                base = torch.full((V, H), 0.5, device=dev) if accumulate else None
+                dh, dw = ops.lmhead_backward(hd, wd, ld, lse, ent, gl, ge, chunk_tokens=chunk, saved_logits=zbuf,
+                                             weight_t=wt, weight_t_ready=wt_ready, dweight=base,
+                                             accumulate_dweight=accumulate)
+                wt_ready = True
+                what = f"saved={saved} chunk={chunk} accumulate={accumulate}"
+                assert_close_rel(dh, dh0, 2 ** -6, "dhidden " + what)
+                assert_close_rel(dw - 0.5 if accumulate else dw, dw0, 2 ** -8, "dweight " + what)
+    assert_close_rel(ops.weight_t_rowmajor(wt, H, V), wd.t().float(), 0.0, "W^T left in the caller's buffer")
