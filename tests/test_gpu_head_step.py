@@ -121,11 +121,26 @@ def test_host_copy_of_the_loss_mask_gives_the_same_bits_without_reading_back(dev
               temperature=cfg.temperature, cu_seqlens_host=cu.tolist(), keep_logits_chunk=keep)
     a = grpo_head_step(*args, **kw)
     b = grpo_head_step(*args, loss_mask_host=mask, **kw)
-    for k in ("logprob", "entropy", "dhidden", "dweight", "sums", "g_logprob"):
-        assert torch.equal(a[k], b[k]), k
-    assert a["rows_projected_bwd"] == b["rows_projected_bwd"] == int(mask.sum())
     lean = grpo_head_step(*args, loss_mask_host=mask, skip_masked_forward=True, **kw)
-    assert torch.equal(lean["dweight"], grpo_head_step(*args, skip_masked_forward=True, **kw)["dweight"])
+    lean_dev = grpo_head_step(*args, skip_masked_forward=True, **kw)
+    assert a["rows_projected_bwd"] == b["rows_projected_bwd"] == int(mask.sum())
+    # the host copy also lets the chunk bound count the unmasked rows only, so the two calls may cut the
+    # micro-batch differently; with the same cuts every output has the same bits, otherwise the per-token
+    # outputs do and the gradients differ by the fp32 summation order over the chunks
+    same_cuts = a["token_chunks"] == b["token_chunks"]
+    for k in ("logprob", "entropy", "g_logprob"):
+        assert torch.equal(a[k], b[k]), k
+    for k in ("dhidden", "dweight", "sums"):
+        if same_cuts:
+            assert torch.equal(a[k], b[k]), k
+        else:
+            assert_close_rel(b[k], a[k], 2 ** -7 if k == "dhidden" else 1e-5, k)
+    if lean["token_chunks"] == lean_dev["token_chunks"]:
+        assert torch.equal(lean["dweight"], lean_dev["dweight"])
+    else:
+        assert_close_rel(lean["dweight"], lean_dev["dweight"], 1e-5, "lean dW")
+    if keep >= T:
+        assert same_cuts
 
 
 def test_kept_logits_backward_equals_recompute(dev):
