@@ -29,7 +29,7 @@ sys.path.insert(0, ROOT)
 
 from chatlearn_amd import _lib, ops, synthetic  # noqa: E402
 from chatlearn_amd._lib import LOSS_GRPO, LOSS_GSPO  # noqa: E402
-from chatlearn_amd.fused import DEFAULT_KEEP_LOGITS_TOKENS, grpo_head_step, head_step_chunks  # noqa: E402
+from chatlearn_amd.fused import default_keep_rows, grpo_head_step, head_step_chunks  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3
@@ -326,7 +326,7 @@ def gemm_kernels(w, keep, reps=3):
     whole backward of the chunk and the backward without that output (what remains in either is the
     d(logits) pass and a transpose)."""
     cfg = w.cfg
-    chunks = head_step_chunks(w.T, keep, cfg.loss == "gspo", w.cu_host, w.mask_host)
+    chunks = head_step_chunks(w.T, keep, cfg.loss == "gspo", w.cu_host, w.mask_host, shape=(cfg.H, cfg.V))
     lo, hi = max(chunks, key=lambda c: c[1] - c[0])
     n = hi - lo
     dev = w.device
@@ -582,7 +582,7 @@ def other_config(name, device, steps, warmup):
     cfg = synthetic.CONFIGS[name]
     w = Workload(cfg, device).tensors().finish()
     train = cfg.loss is not None
-    keep = DEFAULT_KEEP_LOGITS_TOKENS if train else None
+    keep = default_keep_rows(cfg.V, cfg.dtype) if train else None
     dweight = torch.zeros(cfg.V, cfg.H, dtype=torch.float32, device=device) if train else None
     dt, stages, out = time_step(w, keep, dweight, steps, warmup)
     rec = step_record(w, keep, dt, stages, out)
@@ -628,8 +628,9 @@ def main():
                     help="also leave rows whose loss mask is zero out of the forward (their per-token outputs become zero)")
     ap.add_argument("--no-skip-masked", action="store_true",
                     help="run the backward on every row, also those whose loss mask is zero")
-    ap.add_argument("--keep-logits-chunk", type=int, default=DEFAULT_KEEP_LOGITS_TOKENS,
-                    help="tokens per chunk whose logits the forward keeps for the backward (0: recompute)")
+    ap.add_argument("--keep-logits-chunk", type=int, default=-1,
+                    help="rows per chunk whose logits the forward keeps for the backward (0: recompute; "
+                         "-1: the library's default, a bound in bytes)")
     args = ap.parse_args()
     if args.lean:
         args.no_cpu_baseline = args.no_unfused = args.no_variants = args.no_sweep = args.no_other_configs = True
@@ -645,6 +646,8 @@ def main():
     T = w.T
     train = cfg.loss is not None
     dweight = torch.zeros(cfg.V, cfg.H, dtype=torch.float32, device=dev) if train else None
+    if args.keep_logits_chunk < 0:
+        args.keep_logits_chunk = default_keep_rows(cfg.V, cfg.dtype)
     keep = args.keep_logits_chunk if (train and args.keep_logits_chunk > 0) else None
 
     if args.copy_calibration:

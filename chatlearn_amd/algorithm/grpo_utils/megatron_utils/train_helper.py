@@ -8,7 +8,9 @@ Of the reference's ``get_batch`` only the packed (THD) branch is mirrored, as
 branch ([1, 1, S, S] attention masks, position-id resets) and ``forward_step`` are
 Megatron plumbing and stay with the caller; the loss functions here start where the
 model has produced ``all_token_logits`` in Megatron's ``[s, b, V]`` (or
-``[total_nnz, 1, V]``) layout.
+``[total_nnz, 1, V]``) layout - or, through ``compute_all_losses_from_hidden`` /
+``logprobs_from_hidden``, one step earlier: at the decoder's final hidden states, before the
+output layer, so that the logits are never written out.
 """
 from dataclasses import dataclass
 from typing import Any, Dict, Optional
@@ -16,7 +18,8 @@ from typing import Any, Dict, Optional
 import torch
 
 from .... import ops
-from ....bert_padding import pad_input
+from ....bert_padding import index_first_axis, pad_input
+from ....fused import AUTO, fused_linear_logprob_entropy
 from ...._lib import LOSS_GRPO, LOSS_GSPO
 from ..trainer_utils import _StatsFromLogits
 
@@ -75,11 +78,37 @@ def get_batch_packed(data_b: Dict[str, Any], is_training: bool, *, eod: int, tp_
         _, loss_mask = ops.shift_labels(None, loss_mask, zero_last=False)      # roll by -1 along the row
         input_data.update({
             "all_token_loss_mask": loss_mask,
+            # the same rolled mask per packed token, built on the host from the host-side inputs: lets the
+            # fused head find the rows that carry a gradient without reading anything back
+            "packed_loss_mask_host": _packed_loss_mask_host(data_b, seqlen, tp_size * cp_size * 2) if cp_size == 1 else None,
             "advantages": data_b["advantages"],
             "ref_logprobs": data_b["ref_logprobs"].float().to(device),
             "old_logprobs": data_b["old_logprobs"].float().to(device),
         })
     return input_data
+
+
+def _packed_loss_mask_host(data_b, seqlen: int, align: int) -> torch.Tensor:
+    """CPU int32 [total padded tokens]: the training loss mask (response positions, or ``data_b['loss_mask']``)
+    rolled left by one along its [mbs, seqlen] row, then laid out like the packed token row: sequence after
+    sequence, each padded with zeros to a multiple of ``align``."""
+    pl = [int(x) for x in data_b["prompt_token_length"]]
+    rl = [int(x) for x in data_b["response_token_length"]]
+    if "loss_mask" in data_b:
+        m = data_b["loss_mask"].detach().cpu().to(torch.int32)
+    else:
+        m = torch.zeros(len(pl), seqlen, dtype=torch.int32)
+        for i, (p, r) in enumerate(zip(pl, rl)):
+            m[i, p:p + r] = 1
+    m = torch.roll(m, shifts=-1, dims=1)
+    rows = []
+    for i, (p, r) in enumerate(zip(pl, rl)):
+        padded = (p + r + align - 1) // align * align
+        row = torch.zeros(padded, dtype=torch.int32)
+        n = min(padded, seqlen)
+        row[:n] = m[i, :n]
+        rows.append(row)
+    return torch.cat(rows) if rows else torch.zeros(0, dtype=torch.int32)
 
 
 def language_model_logprob(labels: torch.Tensor, logits: torch.Tensor) -> torch.Tensor:
@@ -142,17 +171,10 @@ def _batch_rows(x: torch.Tensor, module_args, training_inputs):
     return reduce_from_context_parallel_region(x, module_args.packing, training_inputs)
 
 
-def _compute_all_losses(module_args, model, all_token_logits: torch.Tensor, labels: torch.Tensor,
-                        training_inputs: Dict[str, Any]) -> Dict[str, torch.Tensor]:
-    """The per-token loss dict of one micro-batch (reference train_helper.py:465-547): keys ``pg_loss``,
-    ``entropy_loss``, ``kl_loss`` and, for the sequence-level policy, the three clip flags twice (summed and
-    sample-averaged by ``loss_func``).  ``model`` is unused: the reference only reaches through it for the
-    cross entropy, which here is the softmax-statistics kernel on the given logits."""
-    del model
+def _loss_dict(module_args, logprob: torch.Tensor, entropy: torch.Tensor,
+               training_inputs: Dict[str, Any]) -> Dict[str, torch.Tensor]:
+    """The loss dict from the [b, s] logprob (carrying the gradient) and the detached [b, s] entropy."""
     gspo = bool(module_args.use_group_sequence_policy)
-    logprob = _batch_rows(language_model_logprob(labels, all_token_logits), module_args, training_inputs)
-    entropy = _batch_rows(entropy_from_tensor_parallel_logits(all_token_logits).permute(1, 0), module_args,
-                          training_inputs)
     adv = torch.tensor(training_inputs["advantages"]).to(logprob.device)      # dtype rule of loss_gallery.py:19,53
     clips = {k: getattr(module_args, k) for k in ("diff_clip_ratio", "pos_clip_ratio", "neg_clip_ratio",
                                                   "final_clip_ratio")}
@@ -166,6 +188,78 @@ def _compute_all_losses(module_args, model, all_token_logits: torch.Tensor, labe
         out.update(zip(names, flags))
         out.update(zip((n + '_sample_average' for n in names), flags))
     return out
+
+
+def _compute_all_losses(module_args, model, all_token_logits: torch.Tensor, labels: torch.Tensor,
+                        training_inputs: Dict[str, Any]) -> Dict[str, torch.Tensor]:
+    """The per-token loss dict of one micro-batch (reference train_helper.py:465-547): keys ``pg_loss``,
+    ``entropy_loss``, ``kl_loss`` and, for the sequence-level policy, the three clip flags twice (summed and
+    sample-averaged by ``loss_func``).  ``model`` is unused: the reference only reaches through it for the
+    cross entropy, which here is the softmax-statistics kernel on the given logits."""
+    del model
+    logprob = _batch_rows(language_model_logprob(labels, all_token_logits), module_args, training_inputs)
+    entropy = _batch_rows(entropy_from_tensor_parallel_logits(all_token_logits).permute(1, 0), module_args,
+                          training_inputs)
+    return _loss_dict(module_args, logprob, entropy, training_inputs)
+
+
+def _token_row_mask(module_args, training_inputs: Dict[str, Any], s: int, b: int):
+    """(device mask, host mask) per row of the flattened [s * b, H] hidden states, from the [B, S] training
+    mask: rows where it is zero get a zero upstream gradient through ``loss_func`` (which multiplies every
+    entry by the mask, train_helper.py:451-455).  Packed rows are looked up through ``indices``."""
+    mask = training_inputs['all_token_loss_mask']
+    if module_args.packing:
+        host = training_inputs.get("packed_loss_mask_host")
+        if host is not None and host.numel() == s * b:
+            return None, host
+        B, S = training_inputs['ori_batch_size'], training_inputs['ori_seq_len']
+        wide = mask.new_zeros(B, S)
+        wide[:, :mask.shape[1]] = mask[:, :S]
+        return index_first_axis(wide.reshape(B * S, 1).to(torch.int32), training_inputs['indices']).reshape(-1), None
+    wide = mask.new_zeros(b, s)
+    wide[:, :mask.shape[1]] = mask[:, :s]
+    return wide.transpose(0, 1).reshape(-1).to(torch.int32), None
+
+
+def compute_all_losses_from_hidden(module_args, hidden: torch.Tensor, output_weight: torch.Tensor,
+                                   labels: torch.Tensor, training_inputs: Dict[str, Any], *, temperature: float = 1.0,
+                                   dweight_buffer: Optional[torch.Tensor] = None, keep_logits_rows=AUTO,
+                                   skip_masked_rows: bool = True) -> Dict[str, torch.Tensor]:
+    """``_compute_all_losses`` with the output layer folded in (reference train_helper.py:465-547 together
+    with the model's ``output_layer`` call that produces its logits, :585-594): ``hidden`` is what the
+    decoder hands to the output layer at ``post_process``, ``[s, b, H]`` or ``[total_nnz, 1, H]``, and
+    ``output_weight`` the ``[V, H]`` weight of that layer.  The same dict comes back - ``pg_loss`` carrying
+    the gradient to ``hidden`` and ``output_weight`` through the fused backward, ``entropy_loss`` detached
+    (the reference's entropy defines no backward, :605-635), ``kl_loss`` and the sequence-level clip flags -
+    and goes into ``loss_func`` unchanged; the ``[*, V]`` logits are never written out.
+
+    ``skip_masked_rows``: ``loss_func`` multiplies every entry by ``all_token_loss_mask``, so rows outside
+    the mask get an exactly zero gradient; their logits are then not kept and the backward leaves them out.
+    Pass False when the loss dict is consumed by something that does not apply the mask.
+    ``dweight_buffer`` (fp32 [V, H], e.g. the weight's ``main_grad``) receives ``+= dW``."""
+    s, b, H = hidden.shape
+    flat_labels = labels.transpose(0, 1).reshape(-1)
+    dev_mask = host_mask = None
+    if skip_masked_rows:
+        dev_mask, host_mask = _token_row_mask(module_args, training_inputs, s, b)
+    lp, ent = fused_linear_logprob_entropy(hidden.reshape(s * b, H), output_weight, flat_labels,
+                                           temperature=temperature, need_entropy=True, dweight_buffer=dweight_buffer,
+                                           keep_logits_rows=keep_logits_rows, loss_mask=dev_mask,
+                                           loss_mask_host=host_mask)
+    logprob = _batch_rows(lp.reshape(s, b).transpose(0, 1), module_args, training_inputs)
+    entropy = _batch_rows(ent.detach().reshape(s, b).permute(1, 0), module_args, training_inputs)
+    return _loss_dict(module_args, logprob, entropy, training_inputs)
+
+
+def logprobs_from_hidden(module_args, hidden: torch.Tensor, output_weight: torch.Tensor, labels: torch.Tensor,
+                         inputs: Dict[str, Any], *, temperature: float = 1.0) -> torch.Tensor:
+    """The no-grad branch of the reference's ``forward_step`` (train_helper.py:585-600): with labels the
+    model returns -cross entropy per token, re-padded to [B, S]; here from the hidden states."""
+    s, b, H = hidden.shape
+    with torch.no_grad():
+        lp, *_ = ops.lmhead_forward(hidden.reshape(s * b, H), output_weight, labels.transpose(0, 1).reshape(-1),
+                                    temperature, need_entropy=False)
+    return _batch_rows(lp.reshape(s, b).transpose(0, 1), module_args, inputs)
 
 
 class _MaskedSums(torch.autograd.Function):
@@ -196,7 +290,8 @@ BACKPROP_KEYS = ('pg_loss',)     # train_helper.py:441
 
 def loss_func(inputs: Dict, losses: Dict[str, torch.Tensor]):
     """(loss to back-propagate, number of unmasked tokens, report) from the per-token loss dict
-    (reference train_helper.py:426-463): every entry is summed under ``all_token_loss_mask`` (a 0/1 mask),
+    (reference train_helper.py:426-463): every entry is summed under ``all_token_loss_mask`` (zeros and ones,
+    as every mask the trainers build; it travels to the kernel as int32),
     the ``*_sample_average`` entries are divided by (1e-5 + number of unmasked tokens), only ``pg_loss``
     keeps its gradient.  All reductions run in one kernel launch."""
     names = list(losses)
@@ -204,7 +299,7 @@ def loss_func(inputs: Dict, losses: Dict[str, torch.Tensor]):
     averaged = tuple(name.endswith('_sample_average') for name in names)
     sums, count = _MaskedSums.apply(inputs["all_token_loss_mask"], grad_slots, averaged,
                                     *(losses[name] for name in names))
-    report = {name: sums[j].detach() for j, name in enumerate(names)}
+    report = {name: sums[j].detach().clone() for j, name in enumerate(names)}
     total = 0
     for j, name in enumerate(names):
         if name in BACKPROP_KEYS:

@@ -14,7 +14,7 @@ from typing import Any, Callable, Dict, List, Optional
 import torch
 
 from ... import ops
-from ...fused import DEFAULT_KEEP_LOGITS_TOKENS, grpo_head_step
+from ...fused import AUTO, grpo_head_step
 from .trainer_utils import (batching, generate_loss_mask_position_ids, split_and_unpadding, split_microbatch,
                             unpad_input)
 
@@ -29,7 +29,7 @@ class PolicyStep:
                  module_args: Optional[Dict[str, Any]] = None, packing: bool = False, max_token_in_seq: int = 32768,
                  train_micro_batch_size: int = 1, generate_micro_batch_size: int = 1, trainable: bool = True,
                  fsdp_size: int = 1, temperature: float = 1.0, dweight_buffer: Optional[torch.Tensor] = None,
-                 keep_logits_chunk: Optional[int] = DEFAULT_KEEP_LOGITS_TOKENS):
+                 keep_logits_chunk=AUTO):
         self.backbone = backbone
         self.weight = lm_head_weight
         self.module_args = dict(_DEFAULT_ARGS)

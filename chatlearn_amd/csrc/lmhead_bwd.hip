@@ -307,9 +307,11 @@ struct GemmParams {
 // Addresses of a 256 x 256 output tile for the accumulator layout: a range-checked buffer descriptor over
 // the tile's valid rows, one per-lane byte offset per 32-wide block of the lane dimension, and an offset
 // per accumulator register (kMContig: per register quad, a compile-time constant; otherwise a uniform
-// multiple of the row pitch).  Elements outside the tile fall outside the descriptor or are skipped as a
-// whole quad (M extents are multiples of 64 here): loads of them give 0 and stores are dropped, so no
-// per-element branch or 64-bit address is needed.
+// multiple of the row pitch, handed to the instruction as its scalar offset).  Along the lane dimension
+// (n) elements outside the tile get a per-lane offset far outside the descriptor: loads of them give 0
+// and stores are dropped.  Along the register dimension (m) nothing relies on the range check, because the
+// scalar offset is not part of it: kMContig skips whole quads (its M extents are multiples of 8), and the
+// other orientation tests every row against the tile's valid rows unless the tile is a full one.
 template <typename T, typename OutT, bool kMContig>
 struct TileAddr {
   using Tile = HeadTile<T>;
@@ -317,6 +319,7 @@ struct TileAddr {
   __amdgpu_buffer_rsrc_t rsrc;
   int voff[Tile::NI];
   int row_bytes, m_first, a_rows;
+  int row_lim;   // valid rows from this lane's first row on: register with row offset dm is inside iff dm < row_lim
   __device__ __forceinline__ TileAddr(OutT* base, int64_t ld, int m0, int n0, int a_rows_, int b_rows) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -324,6 +327,7 @@ struct TileAddr {
     row_bytes = (int)(ld * (int64_t)ES);
     m_first = wm * Tile::WM;
     a_rows = a_rows_;
+    row_lim = a_rows_ - (m_first + 4 * (lane >> 5));
     const int rows = kMContig ? b_rows : a_rows_, cols = kMContig ? a_rows_ : b_rows;
     const int bytes = rows > 0 ? (rows - 1) * row_bytes + cols * ES : 0;
     OutT* origin = kMContig ? base + (int64_t)n0 * ld + m0 : base + (int64_t)m0 * ld + n0;
@@ -341,6 +345,9 @@ struct TileAddr {
     return kMContig ? dm * ES : dm * row_bytes;
   }
   __device__ __forceinline__ bool quad_ok(int mi, int q) const { return m_first + mi * 32 + 8 * q < a_rows; }
+  // row of register r of block row mi, relative to this lane's first row
+  __device__ static __forceinline__ int row_delta(int mi, int r) { return mi * 32 + 8 * (r >> 2) + (r & 3); }
+  __device__ __forceinline__ bool full_rows() const { return a_rows == Tile::BM; }
 };
 
 __device__ __forceinline__ float elem_load(const __amdgpu_buffer_rsrc_t& rsrc, int voff, int soff, float*) {
@@ -378,6 +385,7 @@ __device__ __forceinline__ void quad_store(const f32x16& a, int q, const __amdgp
 template <typename T, typename OutT, bool kMContig, typename AccT>
 __device__ __forceinline__ void tile_load(const TileAddr<T, OutT, kMContig>& at, AccT& acc) {
   using Tile = HeadTile<T>;
+  const bool full = at.full_rows();   // uniform over the workgroup
 #pragma unroll
   for (int ni = 0; ni < Tile::NI; ++ni)
 #pragma unroll
@@ -386,10 +394,15 @@ __device__ __forceinline__ void tile_load(const TileAddr<T, OutT, kMContig>& at,
       for (int q = 0; q < 4; ++q) {
         if (!at.quad_ok(mi, q)) continue;
         if (kMContig) quad_load(acc[mi][ni], q, at.rsrc, at.voff[ni] + at.reg_off(mi, 4 * q), (OutT*)nullptr);
-        else {
+        else if (full) {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             acc[mi][ni][4 * q + i] = elem_load(at.rsrc, at.voff[ni], at.reg_off(mi, 4 * q + i), (OutT*)nullptr);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (at.row_delta(mi, 4 * q + i) < at.row_lim)
+              acc[mi][ni][4 * q + i] = elem_load(at.rsrc, at.voff[ni], at.reg_off(mi, 4 * q + i), (OutT*)nullptr);
         }
       }
 }
@@ -397,6 +410,7 @@ __device__ __forceinline__ void tile_load(const TileAddr<T, OutT, kMContig>& at,
 template <typename T, typename OutT, bool kMContig, typename AccT>
 __device__ __forceinline__ void tile_store(const TileAddr<T, OutT, kMContig>& at, const AccT& acc) {
   using Tile = HeadTile<T>;
+  const bool full = at.full_rows();   // uniform over the workgroup
 #pragma unroll
   for (int ni = 0; ni < Tile::NI; ++ni)
 #pragma unroll
@@ -405,10 +419,15 @@ __device__ __forceinline__ void tile_store(const TileAddr<T, OutT, kMContig>& at
       for (int q = 0; q < 4; ++q) {
         if (!at.quad_ok(mi, q)) continue;
         if (kMContig) quad_store(acc[mi][ni], q, at.rsrc, at.voff[ni] + at.reg_off(mi, 4 * q), (OutT*)nullptr);
-        else {
+        else if (full) {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             elem_store(acc[mi][ni][4 * q + i], at.rsrc, at.voff[ni], at.reg_off(mi, 4 * q + i), (OutT*)nullptr);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (at.row_delta(mi, 4 * q + i) < at.row_lim)
+              elem_store(acc[mi][ni][4 * q + i], at.rsrc, at.voff[ni], at.reg_off(mi, 4 * q + i), (OutT*)nullptr);
         }
       }
 }
@@ -554,6 +573,36 @@ __global__ __launch_bounds__(256) void transpose_block_kernel(const T* __restric
   }
 }
 
+// K ranges per tile that fill `cus` CUs best (1 = no split): work items = tiles x ranges, and a launch
+// takes ceil(items / cus) rounds.  At most kMaxKSplit ranges, each at least 8 slabs long and none empty,
+// and at most what `partial_bytes` can hold of fp32 partial tiles.
+constexpr int kMaxKSplit = 16;
+static int pick_k_split(int tiles, int M, int N, int K, int slab, size_t partial_bytes, int cus) {
+  int best = 1;
+  double best_eff = 0.0;
+  for (int s = 1; s <= kMaxKSplit; ++s) {
+    if (s > 1) {
+      if ((size_t)s * M * N * sizeof(float) > partial_bytes || K / s < 8 * slab) break;
+      const int64_t per = round_up64((K + s - 1) / s, slab);
+      if ((int64_t)(s - 1) * per >= K) continue;     // rounding the range up to whole slabs would leave the last one empty
+    }
+    const long units = (long)tiles * s;
+    const double eff = (double)units / (double)(((units + cus - 1) / cus) * cus);
+    if (eff > best_eff + 0.04) { best_eff = eff; best = s; }   // a split must buy more than 4 % to be worth its extra pass
+  }
+  return best;
+}
+
+// Bytes of fp32 split-K partials the dhidden GEMM of `rows` tokens wants (planned for a 256-CU device, so
+// that the workspace size does not depend on the device in use; a launch takes fewer ranges if they do not fit).
+static size_t dhidden_partial_bytes(int64_t rows, int64_t H, int64_t ldv, int slab) {
+  if (rows <= 0) return 0;
+  const int tiles = (int)(((H + 255) / 256) * ((rows + 255) / 256));
+  const size_t cap = (size_t)1 << 30;
+  const int s = pick_k_split(tiles, (int)H, (int)rows, (int)ldv, slab, cap, 256);
+  return s > 1 ? (size_t)s * rows * H * sizeof(float) : 0;
+}
+
 struct BwdPlan {
   int64_t ldv;        // K extent of dz / WT (V rounded up to 64)
   int64_t chunk;      // tokens per chunk (multiple of 256 unless >= T)
@@ -576,7 +625,11 @@ static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chun
   pl.off_hidt = off; off += align_up(Hb * pl.ldt * es, 256);
   pl.off_dz = off;   off += saved ? 0 : align_up(Cb * pl.ldv * es, 256);
   pl.off_dzt = off;  off += align_up(Vb * pl.ldt * es, 256);
-  pl.part_bytes = align_up((size_t)4 * chunk * H * sizeof(float), 256);   // split-K partials of dhidden
+  // split-K partials of dhidden: what a full chunk and the shorter last chunk want
+  const int slab = (int)(kRowBytes / es);
+  const size_t part_full = dhidden_partial_bytes(chunk, H, pl.ldv, slab);
+  const size_t part_last = dhidden_partial_bytes(T % chunk, H, pl.ldv, slab);
+  pl.part_bytes = align_up(part_full > part_last ? part_full : part_last, 256);
   pl.off_part = off; off += pl.part_bytes;
   pl.total = off;
   return pl;
@@ -593,20 +646,6 @@ static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, s
   return lo * 256;
 }
 
-// K ranges per tile that fill the device's CUs best (1 = no split); at most what `partial_bytes` can hold.
-static int pick_k_split(int tiles, int M, int N, int K, int slab, size_t partial_bytes) {
-  const int cus = device_cu_count();
-  int best = 1;
-  double best_eff = 0.0;
-  for (int s = 1; s <= 4; ++s) {
-    if (s > 1 && ((size_t)s * M * N * sizeof(float) > partial_bytes || K / s < 8 * slab)) break;
-    const long units = (long)tiles * s;
-    const double eff = (double)units / (double)(((units + cus - 1) / cus) * cus);
-    if (eff > best_eff + 0.04) { best_eff = eff; best = s; }   // a split must buy more than 4 % to be worth its extra pass
-  }
-  return best;
-}
-
 template <typename T, typename OutT, bool kMContig>
 static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, int64_t b_kslabs, int N, int K, void* C,
                        int64_t ldc, int accumulate, hipStream_t stream, float* partial = nullptr,
@@ -620,13 +659,13 @@ static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, in
   g.n_mt = (M + 255) / 256; g.n_nt = (N + 255) / 256;
   g.accumulate = accumulate;
   const int slab = Tile::kSlabK;
-  g.k_split = partial ? pick_k_split(g.n_mt * g.n_nt, M, N, K, slab, partial_bytes) : 1;
+  const int cus = device_cu_count();
+  g.k_split = (partial && partial_bytes) ? pick_k_split(g.n_mt * g.n_nt, M, N, K, slab, partial_bytes, cus) : 1;
   g.k_per_split = g.k_split > 1 ? (int)round_up64((K + g.k_split - 1) / g.k_split, slab) : K;
   g.partial = partial;
   // Many more tiles than CUs and no K split: let one workgroup per CU walk runs of tiles instead of
   // launching one workgroup per tile.
   const int n_fixed = kMContig ? g.n_mt : g.n_nt, n_moving = kMContig ? g.n_nt : g.n_mt;
-  const int cus = device_cu_count();
   g.n_walk = 0;
   if (g.k_split == 1 && n_fixed <= cus && g.n_mt * g.n_nt >= 4 * cus && K >= 2 * slab) {
     g.n_walk = cus / n_fixed;

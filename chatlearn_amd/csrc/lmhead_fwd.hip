@@ -70,6 +70,12 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
   if (item >= p.n_tb * p.n_split) return;
   int vs, tb;
   grouped_tile(item, p.n_split, p.n_tb, 4, vs, tb);
+  if (STORE_Z && sizeof(typename KeptLogit<T>::type) == 2) {
+    // Kept logits are IEEE half: a raw logit beyond the half range must stay finite (the largest half),
+    // or the softmax the backward rebuilds from it would be inf/NaN.  The wave's FP16_OVFL mode bit
+    // (MODE register, bit 23) makes every conversion to half clamp instead of overflowing to infinity.
+    __builtin_amdgcn_s_setreg(1 | (23 << 6) | (0 << 11), 1);
+  }
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;

@@ -22,7 +22,23 @@ from . import ops
 from ._lib import LOSS_GRPO, LOSS_GSPO
 
 
-DEFAULT_KEEP_LOGITS_TOKENS = 8192   # tokens whose logits one chunk keeps for its backward (2.5 GB at a 152k vocabulary)
+# Memory one chunk's kept logits may take (they are turned into d(logits) in place; the backward's transposed
+# copy takes as much again).  The bound is on bytes, whatever the hidden size: 17408 rows of a 152k
+# vocabulary, 20736 rows of a 129k one, in 16-bit elements.
+DEFAULT_KEEP_LOGITS_BYTES = 5 << 30
+AUTO = "auto"
+
+
+def default_keep_rows(V: int, dtype) -> int:
+    """Rows whose logits fit DEFAULT_KEEP_LOGITS_BYTES: a multiple of 256 (the kept-logits buffer is cut
+    into blocks of 256 rows), at least 256."""
+    es = torch.empty(0, dtype=dtype).element_size()
+    rows = DEFAULT_KEEP_LOGITS_BYTES // (ops.saved_logits_ld(V) * es)
+    return max(256, rows // 256 * 256)
+
+
+def _resolve_keep(keep, V, dtype):
+    return default_keep_rows(V, dtype) if isinstance(keep, str) and keep == AUTO else keep
 
 
 def _nonzero_rows(mask: torch.Tensor) -> torch.Tensor:
@@ -92,34 +108,51 @@ def _live_rows_from_host_mask(mask_host: torch.Tensor, chunks, device):
     return [(local_d[a:b], map_d[lo:hi]) for (a, b), (lo, hi) in zip(counts, chunks)]
 
 
+def _host_live_rows(mask_host, T):
+    """Ascending positions of the nonzero entries of a host copy of the loss mask (numpy int64)."""
+    if not isinstance(mask_host, torch.Tensor) or mask_host.is_cuda:
+        raise TypeError("loss_mask_host must be a CPU tensor")
+    if mask_host.numel() != T:
+        raise ValueError(f"loss_mask_host has {mask_host.numel()} entries for {T} tokens")
+    return np.flatnonzero(mask_host.reshape(-1).numpy() != 0).astype(np.int64)
+
+
 class _FusedHead(torch.autograd.Function):
+    """Rows that carry a gradient ("live": all rows, or the unmasked ones when the caller hands in the loss
+    mask) are split in two: the first ``keep_rows`` of them keep their logits in the forward, and their
+    backward runs from those; the others are recomputed in the backward.  Both parts add into one dW."""
+
     @staticmethod
-    def forward(ctx, hidden, weight, labels, temperature, need_entropy, dweight_buffer, keep_rows, row_mask):
+    def forward(ctx, hidden, weight, labels, temperature, need_entropy, dweight_buffer, keep_rows, row_mask, mask_host):
         T = hidden.shape[0]
-        zbuf = live = row_map = None
+        dev = hidden.device
+        zbuf = row_map = None
+        live = None            # device int64 positions of the live rows; None: every row
+        n_live = T
         if keep_rows is not None and T > 0:
-            if row_mask is not None:
-                # rows outside the mask get a zero upstream gradient whatever their logits are:
-                # keep logits only for the others and run the backward on that compact set
-                live = _nonzero_rows(row_mask)
-            rows = T if live is None else int(live.numel())
-            if rows > keep_rows:
-                live = None                  # more rows than may be kept: the backward recomputes its logit tiles
-            elif rows > 0:
-                zbuf = ops.saved_logits_buffer(rows, weight.shape[0], hidden.dtype, hidden.device)
-                if live is not None:
-                    row_map = torch.full((T,), -1, dtype=torch.int32, device=hidden.device)
-                    row_map[live] = torch.arange(live.numel(), dtype=torch.int32, device=hidden.device)
+            if mask_host is not None:
+                live_h = _host_live_rows(mask_host, T)          # no device value is read back
+                n_live = int(live_h.size)
+                live = _upload(torch.from_numpy(live_h), dev) if n_live else torch.empty(0, dtype=torch.int64, device=dev)
+            elif row_mask is not None:
+                live = _nonzero_rows(row_mask)                  # one host round trip for the count
+                n_live = int(live.numel())
+        n_kept = 0 if keep_rows is None else min(int(keep_rows), n_live)
+        if n_kept > 0:
+            zbuf = ops.saved_logits_buffer(n_kept, weight.shape[0], hidden.dtype, dev)
+            if live is not None:
+                row_map = torch.full((T,), -1, dtype=torch.int32, device=dev)
+                row_map[live[:n_kept]] = torch.arange(n_kept, dtype=torch.int32, device=dev)
         lp, ent, _, lse = ops.lmhead_forward(hidden, weight, labels, temperature, need_entropy,
-                                             saved_logits=zbuf, saved_row_map=row_map if zbuf is not None else None)
+                                             saved_logits=zbuf, saved_row_map=row_map)
         ctx.save_for_backward(hidden, weight, labels, lse, ent if ent is not None else lse)
         ctx.set_materialize_grads(False)
         ctx.temperature = temperature
         ctx.has_entropy = ent is not None
         ctx.dweight_buffer = dweight_buffer
-        ctx.zbuf, ctx.live = zbuf, live
+        ctx.zbuf, ctx.live, ctx.n_live, ctx.n_kept = zbuf, live, n_live, n_kept
         if ent is None:
-            ent = torch.zeros(0, device=hidden.device)
+            ent = torch.zeros(0, device=dev)
             ctx.mark_non_differentiable(ent)
         return lp, ent
 
@@ -127,9 +160,11 @@ class _FusedHead(torch.autograd.Function):
     def backward(ctx, g_lp, g_ent):
         hidden, weight, labels, lse, ent = ctx.saved_tensors
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        zbuf, live = ctx.zbuf, ctx.live
+        zbuf, live, n_live, n_kept = ctx.zbuf, ctx.live, ctx.n_live, ctx.n_kept
         ctx.zbuf = None                      # the buffer is consumed (overwritten) by this backward
-        none = (None,) * 8
+        if zbuf is None:
+            n_kept = 0                       # a second backward through a retained graph recomputes
+        none = (None,) * 9
         if g_lp is None and g_ent is None:
             return none
         if g_lp is None:
@@ -139,31 +174,45 @@ class _FusedHead(torch.autograd.Function):
         g_ent = g_ent.float().contiguous() if use_ent else None
         ent = ent if use_ent else None
         T = hidden.shape[0]
-        kw = dict(need_dhidden=need_h, need_dweight=need_w, dweight=ctx.dweight_buffer,
-                  accumulate_dweight=ctx.dweight_buffer is not None)
-        if live is None:
-            dh, dw = ops.lmhead_backward(hidden, weight, labels, lse, ent, g_lp, g_ent, ctx.temperature,
-                                         saved_logits=zbuf, **kw)
-        elif live.numel() == 0:
+        dw_buf = ctx.dweight_buffer
+        if n_live == 0:
             dh = torch.zeros_like(hidden) if need_h else None
-            dw = None
-            if need_w and ctx.dweight_buffer is None:
-                dw = torch.zeros(weight.shape, dtype=torch.float32, device=hidden.device)
-        else:
-            pick = lambda x: None if x is None else ops.gather_rows(x.reshape(T, -1), live).reshape(-1)
-            dh_c, dw = ops.lmhead_backward(ops.gather_rows(hidden, live), weight, pick(labels), pick(lse), pick(ent),
-                                           pick(g_lp), pick(g_ent), ctx.temperature, saved_logits=zbuf, **kw)
-            dh = ops.scatter_rows(dh_c, live, T) if need_h else None
+            dw = torch.zeros(weight.shape, dtype=weight.dtype, device=hidden.device) if (need_w and dw_buf is None) else None
+            return (dh, dw) + (None,) * 7
+
+        def part(lo, hi, saved, dweight, accumulate):
+            """Backward of live rows [lo, hi) (in live order): from kept logits, or recomputing them."""
+            if live is None:
+                pick = lambda x: None if x is None else x[lo:hi]
+            else:
+                idx = live[lo:hi]
+                pick = lambda x: None if x is None else ops.gather_rows(x.reshape(T, -1), idx).reshape((hi - lo,) + x.shape[1:])
+            return ops.lmhead_backward(pick(hidden), weight, pick(labels), pick(lse), pick(ent), pick(g_lp), pick(g_ent),
+                                       ctx.temperature, need_dhidden=need_h, need_dweight=need_w, dweight=dweight,
+                                       accumulate_dweight=accumulate, saved_logits=saved)
+
+        dw, acc = dw_buf, dw_buf is not None
+        pieces = []
+        for lo, hi, saved in ((0, n_kept, zbuf), (n_kept, n_live, None)):
+            if hi > lo:
+                dh_p, dw = part(lo, hi, saved, dw, acc)
+                acc = True
+                pieces.append(dh_p)
+        dh = None
+        if need_h:
+            dh_c = pieces[0] if len(pieces) == 1 else torch.cat(pieces, 0)
+            dh = dh_c if live is None else ops.scatter_rows(dh_c, live, T)
         if dw is not None:
             # A caller-supplied fp32 main-grad buffer was accumulated in place; autograd gets no copy.
-            dw = None if ctx.dweight_buffer is not None else dw.to(weight.dtype)
-        return (dh, dw) + (None,) * 6
+            dw = None if dw_buf is not None else dw.to(weight.dtype)
+        return (dh, dw) + (None,) * 7
 
 
 def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, *,
                                  temperature: float = 1.0, need_entropy: bool = True,
                                  dweight_buffer: Optional[torch.Tensor] = None,
-                                 keep_logits_rows: Optional[int] = DEFAULT_KEEP_LOGITS_TOKENS, loss_mask: Optional[torch.Tensor] = None):
+                                 keep_logits_rows=AUTO, loss_mask: Optional[torch.Tensor] = None,
+                                 loss_mask_host: Optional[torch.Tensor] = None):
     """(logprob fp32 [T], entropy fp32 [T]) of ``labels`` under softmax(hidden @ weight.T / temperature).
 
     hidden [T,H] and weight [V,H] share a dtype (bf16 or fp32), labels int64 [T].
@@ -172,39 +221,43 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     without it ``weight.grad`` gets dW cast to the weight dtype, as torch would.
     Leading dimensions of hidden/labels are flattened and restored.
 
-    ``keep_logits_rows``: when a gradient is needed and there are at most this many rows (with
-    ``loss_mask``: unmasked rows), the forward keeps their raw logits (one 16-bit copy for 16-bit inputs, released by the backward) so that the
-    backward does not recompute them; ``None`` or more rows: recompute.  The default bounds the kept
-    logits at 2.5 GB for a 152k vocabulary; a caller that wants the fast path for a larger micro-batch
-    either raises it or runs the head chunk by chunk (forward, loss, backward per chunk), which is what
-    ``grpo_head_step`` does.  ``loss_mask`` (same shape as
-    ``labels``) is a promise that rows where it is zero receive a zero upstream gradient - true
-    of the reference's loss, which multiplies by this mask (policy_trainer.py:259-283): their
-    logits are then not kept and the backward runs on the other rows only.
+    ``keep_logits_rows``: when a gradient is needed, the forward keeps the raw logits of up to this many
+    rows (one 16-bit copy for 16-bit inputs, released by the backward) so that the backward does not
+    recompute them; rows beyond the bound are recomputed in the backward, tile by tile, and both parts
+    add into one dW.  ``"auto"`` (the default) bounds the kept logits at ``DEFAULT_KEEP_LOGITS_BYTES``;
+    ``None`` keeps nothing.  A caller that owns the training loop can instead run the head chunk by
+    chunk (forward, loss, backward per chunk), which is what ``grpo_head_step`` does.
+
+    ``loss_mask`` (same shape as ``labels``) is a promise that rows where it is zero receive a zero
+    upstream gradient - true of the reference's loss, which multiplies by this mask
+    (policy_trainer.py:259-283): their logits are then not kept and the backward runs on the other
+    rows only.  ``loss_mask_host`` is a CPU copy of the same mask (the trainer builds the mask on the
+    host anyway): with it the unmasked rows are found on the host and nothing is read back from the
+    device; with the device mask alone, their count costs one host round trip.
     """
     lead = labels.shape
     h2 = hidden.reshape(-1, hidden.shape[-1])
-    T = h2.shape[0]
     needs_grad = torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad)
-    keep = keep_logits_rows if needs_grad else None      # rows whose logits may be kept; None: keep nothing
+    keep = _resolve_keep(keep_logits_rows, weight.shape[0], hidden.dtype) if needs_grad else None
     mask = None
-    if keep is not None and loss_mask is not None:
+    if keep is not None and loss_mask is not None and loss_mask_host is None:
         mask = loss_mask.reshape(-1).to(torch.int32)
     lp, ent = _FusedHead.apply(h2, weight, labels.reshape(-1), float(temperature), bool(need_entropy), dweight_buffer,
-                               keep, mask)
+                               keep, mask, loss_mask_host if keep is not None else None)
     lp = lp.reshape(lead)
     ent = ent.reshape(lead) if need_entropy else None
     return lp, ent
 
 
-def _token_chunks(T, chunk_rows, seq_bounds, live_cum=None):
+def _token_chunks(T, chunk_rows, seq_bounds, live_cum=None, n_ranges=None):
     """[lo, hi) token ranges holding at most ``chunk_rows`` rows each: as few ranges as that allows, and
     of about equal length in tokens (the forward runs on every token of a range; a short last range would
     run all kernels at poor efficiency).  A token counts as a row, unless ``live_cum`` is given (a numpy
     array, live_cum[i] = rows among tokens [0, i) whose logits are kept, i.e. the unmasked ones): then the
     bound is on those.  With ``seq_bounds`` (the host copy of cu_seqlens) every range ends on a sequence
     boundary (a range exceeds ``chunk_rows`` only where a single sequence is larger than it), otherwise
-    on a multiple of 256 tokens where the bound leaves room for that."""
+    on a multiple of 256 tokens where the bound leaves room for that.  ``n_ranges`` asks for that many
+    ranges instead of the fewest (it is raised to the fewest when smaller)."""
     total = T if live_cum is None else int(live_cum[T])
     if chunk_rows is None or chunk_rows >= total or T == 0:
         return [(0, T)]
@@ -245,6 +298,8 @@ def _token_chunks(T, chunk_rows, seq_bounds, live_cum=None):
         if wt(lo) == total:
             lo = T                                                 # a tail without rows rides along
         n += 1
+    if n_ranges is not None:
+        n = max(n, int(n_ranges))
     out, lo = [], 0
     while lo < T:
         left = n - len(out)
@@ -260,11 +315,44 @@ def _token_chunks(T, chunk_rows, seq_bounds, live_cum=None):
     return out
 
 
-def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask_host=None):
+def _launch_cost(chunks, live_cum, H, V, cus=256):
+    """Relative time of the three GEMM-shaped launches of every chunk, in units of one 256 x 256 tile
+    over one K element on one CU: a launch of n work items takes ceil(n / cus) rounds.  Mirrors the
+    library's launch plans (vocabulary splits of the forward, K ranges of the dhidden GEMM, walking
+    workgroups of the dW GEMM); the passes that do not depend on the cuts (d(logits), transposes)
+    are left out, the read of dW's previous contents by every chunk after the first is counted."""
+    n_vt = -(-V // 256)
+    n_ht = -(-H // 256)
+    cost = 0.0
+    for k, (lo, hi) in enumerate(chunks):
+        rows = (hi - lo) if live_cum is None else int(live_cum[hi] - live_cum[lo])
+        n_tb = -(-(hi - lo) // 256)
+        best = None
+        for sp in range(1, min(64, n_vt) + 1):                 # forward: rounds x vocabulary tiles per workgroup
+            tps = -(-n_vt // sp)
+            c = -(-(n_tb * -(-n_vt // tps)) // cus) * tps
+            best = c if best is None else min(best, c)
+        cost += best * H
+        if rows == 0:
+            continue
+        n_rt = -(-rows // 256)
+        tiles = n_ht * n_rt                                    # dhidden: K = V, up to 16 K ranges
+        cost += min(-(-(tiles * s) // cus) * (V / s) for s in range(1, 17))
+        walk = max(1, cus // n_ht)                             # dW: workgroups keep an H tile and walk vocabulary tiles
+        cost += (-(-n_vt // min(walk, n_vt)) if n_vt * n_ht >= 4 * cus else -(-(n_vt * n_ht) // cus)) * rows
+        if k > 0:
+            cost += 0.15 * n_vt * n_ht / cus * 2048            # re-reading dW [V,H] fp32: HBM time in the same unit
+    return cost
+
+
+def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask_host=None, shape=None):
     """The token ranges ``grpo_head_step`` walks: at most ``keep_logits_chunk`` kept rows each.  Only
     unmasked rows keep their logits, so with the mask known on the host (``loss_mask_host``, given when
     masked rows are skipped) the bound counts those; the sequence-level loss needs ranges that end on
-    sequence boundaries (``cu_seqlens``: host list or device tensor, read only when a split is needed)."""
+    sequence boundaries (``cu_seqlens``: host list or device tensor, read only when a split is needed).
+    With ``shape`` = (H, V) the number of ranges is the fewest the bound allows or up to two more,
+    whichever fills the CUs best over the forward and the two backward GEMMs (a launch takes whole
+    rounds of one workgroup per CU; ragged sequence-aligned ranges can leave a round nearly empty)."""
     live_cum = None
     if loss_mask_host is not None and T > 0:
         live_cum = np.concatenate([[0], np.cumsum(loss_mask_host.reshape(-1).numpy() != 0, dtype=np.int64)])
@@ -272,7 +360,19 @@ def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask
     bounds = None
     if keep_logits_chunk is not None and keep_logits_chunk < rows_total and sequence_level:
         bounds = cu_seqlens.tolist() if isinstance(cu_seqlens, torch.Tensor) else list(cu_seqlens)
-    return _token_chunks(T, keep_logits_chunk, bounds, live_cum)
+    fewest = _token_chunks(T, keep_logits_chunk, bounds, live_cum)
+    if shape is None or len(fewest) == 1:
+        return fewest
+    H, V = shape
+    best, best_cost = fewest, _launch_cost(fewest, live_cum, H, V)
+    for extra in (1, 2):
+        cand = _token_chunks(T, keep_logits_chunk, bounds, live_cum, n_ranges=len(fewest) + extra)
+        if len(cand) != len(fewest) + extra:
+            continue
+        c = _launch_cost(cand, live_cum, H, V)
+        if c < 0.98 * best_cost:                                # more ranges must buy more than 2 %
+            best, best_cost = cand, c
+    return best
 
 
 def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages, cu_seqlens, loss_mask, *,
@@ -280,7 +380,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                    pos_clip_ratio=0.2, neg_clip_ratio=0.2, diff_clip_ratio=10, final_clip_ratio=3,
                    kl_coef=0.0, entropy_coef=0.0, temperature=1.0, dweight: Optional[torch.Tensor] = None,
                    accumulate_dweight=False, need_dhidden=True, check_flags=True,
-                   keep_logits_chunk: Optional[int] = DEFAULT_KEEP_LOGITS_TOKENS, cu_seqlens_host=None,
+                   keep_logits_chunk=AUTO, cu_seqlens_host=None,
                    skip_masked_rows=True, skip_masked_forward=False, weight_t_cache: Optional[dict] = None,
                    stage_hook=None, loss_mask_host: Optional[torch.Tensor] = None,
                    workspace_cache: Optional[dict] = None):
@@ -293,7 +393,8 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
 
     ``keep_logits_chunk``: the micro-batch is walked in token chunks that keep the raw logits of at most
     this many rows (one [chunk, V] buffer of 16-bit or fp32 elements, reused chunk after chunk) so that
-    the backward does not recompute them.  Every token counts as a row, except that with
+    the backward does not recompute them; ``"auto"`` (the default) bounds that buffer at
+    ``DEFAULT_KEEP_LOGITS_BYTES``.  Every token counts as a row, except that with
     ``skip_masked_rows`` and ``loss_mask_host`` only the unmasked tokens do (only they are kept).  ``None`` keeps nothing: the
     backward then recomputes the logit tiles from ``hidden`` and ``weight``.  The sequence-level
     loss needs chunks that end on sequence boundaries, so it reads ``cu_seqlens_host`` (or copies
@@ -329,12 +430,15 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     hook = stage_hook or (lambda name: None)
     T = hidden.shape[0]
     V = weight.shape[0]
+    keep_logits_chunk = _resolve_keep(keep_logits_chunk, V, hidden.dtype)
     scale = float(fsdp_size) / float(n_tokens_total)
     mode = LOSS_GSPO if use_group_sequence_policy else LOSS_GRPO
     skip = keep_logits_chunk is not None and loss_mask is not None and skip_masked_rows
+    if loss_mask_host is not None and (loss_mask_host.is_cuda or loss_mask_host.numel() != T):
+        raise ValueError(f"loss_mask_host must be a CPU copy of loss_mask with {T} entries")
     chunks = head_step_chunks(T, keep_logits_chunk, use_group_sequence_policy,
                               cu_seqlens_host if cu_seqlens_host is not None else cu_seqlens,
-                              loss_mask_host if skip else None)
+                              loss_mask_host if skip else None, shape=(hidden.shape[1], V))
     zbuf = None
     rows_of = None
     if skip and loss_mask_host is not None and T > 0:
@@ -452,10 +556,16 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
         sums += res.sums
         flags |= res.flags
     if check_flags:
-        fl = int(flags.item())
+        # one read-back for the reference's three assertions and the host mask's consistency
+        fl, n_masked = (int(x) for x in torch.stack([flags[0].double(), sums[3]]).tolist())
         assert not fl & 1, "pg loss is nan"
         assert not fl & 2, "kl loss ratio has inf values"
         assert not fl & 4, "kl loss ratio has nan values"
+        if rows_of is not None and loss_mask is not None:
+            n_host = int(loss_mask_host.sum())
+            if n_host != n_masked:
+                raise ValueError(f"loss_mask_host sums to {n_host}, the device loss_mask to {n_masked}: "
+                                 "the host copy is stale or laid out differently")
     pg = sums[0] * scale
     kl = sums[1] * scale
     en = sums[2] * scale

@@ -112,7 +112,8 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
     """(logprob, entropy, rowmax, lse), each fp32 [T].  Logits are not materialised unless the caller
     hands in ``saved_logits`` (from ``saved_logits_buffer``) for these T rows, which a following
     ``lmhead_backward`` of the same rows consumes instead of recomputing them.  ``saved_row_map``
-    (int32 [T]) sends token t's logits to row ``map[t]`` of the buffer, or nowhere if negative."""
+    (int32 [T]) sends token t's logits to row ``map[t]`` of the buffer, or nowhere if negative; without
+    a map token t goes to row t, and tokens past the buffer's rows are not kept."""
     hidden = _dev(hidden, "hidden")
     weight = _dev(weight, "weight", hidden.dtype)
     if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
@@ -145,8 +146,8 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
         saved_logits = _dev(saved_logits, "saved_logits", hidden.dtype)
         if saved_logits.dim() != 2 or not saved_logits.is_contiguous():
             raise ValueError("saved_logits must be a contiguous [rows, ld] tensor")
-        if saved_logits.shape[0] % 256 != 0 or (saved_row_map is None and saved_logits.shape[0] < T):
-            raise ValueError("saved_logits must come from saved_logits_buffer with at least T rows")
+        if saved_logits.shape[0] % 256 != 0:
+            raise ValueError("saved_logits must come from saved_logits_buffer (whole blocks of 256 rows)")
         ld_saved = saved_logits.shape[1]
         if saved_row_map is not None:
             saved_row_map = _dev(saved_row_map, "saved_row_map", torch.int32)

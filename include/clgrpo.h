@@ -34,6 +34,15 @@ typedef enum {
 
 typedef enum { CLGRPO_BF16 = 0, CLGRPO_F32 = 1, CLGRPO_F64 = 2, CLGRPO_U8 = 3 /* bool / uint8 flags */ } clgrpo_dtype;
 
+/* major * 100 + minor.  A change of an args struct's layout or of a buffer's meaning raises the major part;
+ * callers compare clgrpo_version() / 100 with the CLGRPO_VERSION / 100 they were built against.
+ *   1.00 -> 2.00: clgrpo_lmhead_fwd_args / clgrpo_lmhead_bwd_args gained saved_rows (must be set whenever
+ *                 saved_logits is); clgrpo_softmax_stats_bwd_args gained lse and entropy; kept logits of 16-bit
+ *                 inputs are IEEE half in the forward's own order; clgrpo_lmhead_fwd_workspace_bytes grew to
+ *                 min(ceil(V / 256), 64) * T * 16.
+ *   2.00 -> 2.01: clgrpo_lmhead_bwd_workspace_bytes sizes the split-K partials by the GEMM's plan (smaller in
+ *                 general); clgrpo_policy_loss_args.megatron (appended) selects the Megatron loss sums. */
+#define CLGRPO_VERSION 201
 int clgrpo_version(void);
 const char* clgrpo_last_error_string(void);
 
@@ -64,7 +73,9 @@ typedef struct {
                               The buffer is opaque to the caller: ceil(rows / 256) * 256 rows of ld_saved elements
                               of sizeof(dtype) bytes.  The forward fills it in the order of its accumulators
                               (32 KB units of 256 rows x 128 bytes of vocabulary, inside a unit 32 x 32 sub-blocks
-                              stored as 16-byte pieces per lane; 16-bit inputs keep their logits as IEEE half);
+                              stored as 16-byte pieces per lane; 16-bit inputs keep their logits as IEEE half, a raw
+                              logit beyond +-65504 as +-65504: the backward's gradients stay finite, but that
+                              token's probabilities are then formed from the saturated value);
                               the backward overwrites every unit in place with d(logits) as the K-blocked operand
                               of its GEMMs: element (row, k) at
                               (((row / 256) * (ld_saved / E) + k / E) * 256 + row % 256) * E + k % E,

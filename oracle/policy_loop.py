@@ -13,7 +13,8 @@ logits [b, s, V].  Everything runs on the CPU with the other oracle modules.
 Pinned by tests/test_policy_loop_cpu.py: a three-sample case worked by hand from the
 reference lines above (micro-batch order with a tie on the bin totals, packed token row,
 indices, position ids, labels that roll across sequence boundaries, shifted training mask,
-N, per-sample record lengths and values, train_stats) with literal expected tables.
+N, per-sample record lengths and values, train_stats) with literal expected tables, and the
+sequence-level (GSPO) variant of the loss by hand-worked sequence ratios on the same case.
 """
 import torch
 import torch.nn.functional as F
@@ -81,7 +82,10 @@ def train_step(model, data_list, *, packing, module_args, **prep):
             logprobs, entropy, inputs["old_logprobs"], inputs["ref_logprobs"], inputs["advantages"],
             inputs["loss_mask"], n_tok, entropy_coef=module_args["entropy_coef"], kl_coef=module_args["kl_coef"],
             pos_clip_ratio=module_args.get("pos_clip_ratio", 0.2), neg_clip_ratio=module_args.get("neg_clip_ratio", 0.2),
-            diff_clip_ratio=module_args.get("diff_clip_ratio", 10), final_clip_ratio=module_args.get("final_clip_ratio", 3))
+            diff_clip_ratio=module_args.get("diff_clip_ratio", 10), final_clip_ratio=module_args.get("final_clip_ratio", 3),
+            # the reference wires the sequence-level surrogate into its Megatron trainer only
+            # (train_helper.py:491-506); on this loop it is the same arithmetic on the same padded rows
+            use_group_sequence_policy=module_args.get("use_group_sequence_policy", False))
         total.backward()
         totals.append(total.detach())
         pg_l.append(parts["pg_loss"]); en_l.append(parts["entropy_loss"]); kl_l.append(parts["kl_loss"])

@@ -68,3 +68,37 @@ def test_chunks_bounded_by_kept_rows():
                     assert not any(lo < x < hi and cum[lo] < cum[x] < cum[hi] for x in bounds)
         if len(ranges) > 1:
             assert rows[-1] > 0 or bounds is not None                                      # no range for a tail without kept rows
+
+
+def test_asked_number_of_ranges_and_launch_cost_choice():
+    from chatlearn_amd.fused import _launch_cost, head_step_chunks
+    # more ranges than the fewest: still a partition, still within the bound
+    assert _token_chunks(1000, 600, None, None, n_ranges=4) == [(0, 256), (256, 512), (512, 768), (768, 1000)]
+    assert len(_token_chunks(1000, 600, None, None, n_ranges=1)) == 2                      # never fewer than the bound needs
+    rng = random.Random(3)
+    for _ in range(500):
+        T = rng.randint(10, 6000)
+        cap = rng.randint(5, 3000)
+        bounds = sorted({0, T} | {rng.randint(1, T) for _ in range(rng.randint(1, 30))}) if rng.random() < 0.5 else None
+        fewest = _token_chunks(T, cap, bounds)
+        for extra in (1, 2):
+            r = _token_chunks(T, cap, bounds, None, n_ranges=len(fewest) + extra)
+            assert r[0][0] == 0 and r[-1][1] == T and all(a[1] == b[0] for a, b in zip(r, r[1:]))
+            assert all(hi > lo for lo, hi in r) and len(r) >= len(fewest)
+            if bounds is None:
+                assert all(hi - lo <= cap for lo, hi in r)
+    # the cost counts whole rounds of one workgroup per CU: 64 token blocks x 4 vocabulary splits fill 256 CUs
+    # (149 tiles each); 65 blocks fill them worse whatever the split (3 splits: 195 workgroups x 198 tiles)
+    H, V = 2048, 151936
+    one, more = _launch_cost([(0, 16384)], None, H, V), _launch_cost([(0, 16640)], None, H, V)
+    assert one / 16384 < more / 16640
+    # a sequence-level micro-batch of 32768 tokens: the bound of 17408 rows allows two ranges; the choice
+    # never takes more than two extra and every range ends on a sequence boundary
+    cu = [0, 5000, 9000, 16000, 21000, 26000, 30000, 32768]
+    import torch
+    mask = torch.ones(32768, dtype=torch.int32)
+    ranges = head_step_chunks(32768, 17408, True, cu, mask, shape=(H, V))
+    assert 2 <= len(ranges) <= 4 and all(hi in cu for _, hi in ranges)
+    assert ranges[0][0] == 0 and ranges[-1][1] == 32768
+    # everything fits one range: one range, whatever the shape
+    assert head_step_chunks(16384, 17408, False, None, None, shape=(4096, V)) == [(0, 16384)]

@@ -161,10 +161,32 @@ def test_autograd_kept_logits_mask_hint_and_second_backward(dev, dtype):
     rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, c_lp, c_ent, 0.8)
     r = RTOL[dtype]
     assert_close_rel(ref_h, rdh, r, "recompute dh")
-    for name, kw in (("kept", {}), ("kept + mask hint", dict(loss_mask=mask.to(dev)))):
+    cases = (("kept", {}), ("kept + mask hint", dict(loss_mask=mask.to(dev))),
+             ("kept + host mask", dict(loss_mask_host=mask)),
+             # more rows carry a gradient than may be kept: the first ones run from kept logits, the rest are
+             # recomputed, and both parts add into one dW
+             ("100 of 300 rows kept, no mask", dict(keep_logits_rows=100)),
+             ("64 unmasked rows kept, the others recomputed", dict(keep_logits_rows=64, loss_mask=mask.to(dev))),
+             ("64 kept, host mask", dict(keep_logits_rows=64, loss_mask_host=mask)),
+             ("256 kept (one block), no mask", dict(keep_logits_rows=256)))
+    assert int(mask.sum()) > 64
+    for name, kw in cases:
         gh, gw = grads(**kw)
         assert_close_rel(gh, rdh, r, name + " dh")
         assert_close_rel(gw, rdw, r, name + " dW")
+        if "mask" in name:
+            assert (gh[mask.to(dev) == 0] == 0).all(), name
+    # the hybrid with a caller's fp32 gradient buffer: both parts add to what it held
+    main_grad = torch.full((V, H), 0.5, device=dev)
+    h = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    lp, ent = fused_linear_logprob_entropy(h, w, labels.to(dev), temperature=0.8, keep_logits_rows=64,
+                                           loss_mask_host=mask, dweight_buffer=main_grad)
+    ((lp * c_lp.to(dev)).sum() + (ent * c_ent.to(dev)).sum()).backward()
+    assert w.grad is None
+    assert_close_rel(main_grad - 0.5, rdw, r, "hybrid dW added to the main-grad buffer")
+    with pytest.raises(ValueError, match="entries"):
+        fused_linear_logprob_entropy(h, w, labels.to(dev), loss_mask_host=mask[:-1])
     (h1, w1), (h2, w2) = grads(retain=True, loss_mask=mask.to(dev))
     assert_close_rel(h2, rdh, r, "second backward dh")
     assert_close_rel(w2, rdw, r, "second backward dW")
@@ -284,3 +306,81 @@ def test_backward_option_combinations_agree(dev):
                 assert_close_rel(dh, dh0, 2 ** -6, "dhidden " + what)
                 assert_close_rel(dw - 0.5 if accumulate else dw, dw0, 2 ** -8, "dweight " + what)
     assert_close_rel(ops.weight_t_rowmajor(wt, H, V), wd.t().float(), 0.0, "W^T left in the caller's buffer")
+
+
+@pytest.mark.parametrize("V", [777, 2100, 2500])
+@pytest.mark.parametrize("accumulate", [False, True])
+@pytest.mark.parametrize("saved", [False, True])
+def test_weight_gradient_never_touches_memory_past_its_last_row(dev, V, accumulate, saved):
+    """dW [V,H] handed in as the front of a larger buffer whose remainder holds a sentinel: a vocabulary that
+    ends inside a 256-row tile (and not on a multiple of 8 rows) must leave every byte after row V alone,
+    whether the GEMM writes dW or adds to it, and on both backward routes."""
+    from chatlearn_amd import ops
+    T, H = 520, 128
+    hidden, weight, labels = _inputs(T, H, V, torch.bfloat16, seed=V, w_std=0.1)
+    g_lp = torch.randn(T, generator=torch.Generator().manual_seed(V + 1))
+    hd, wd, ld, gd = hidden.to(dev), weight.to(dev), labels.to(dev), g_lp.to(dev)
+    guard_rows = 300                                   # more than one whole tile of rows behind the tensor
+    sentinel = 1234.5
+    buf = torch.full(((V + guard_rows) * H,), sentinel, device=dev)
+    dw_view = buf[:V * H].view(V, H)
+    if accumulate:
+        dw_view.fill_(0.25)
+    zbuf = ops.saved_logits_buffer(T, V, torch.bfloat16, dev) if saved else None
+    lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld, saved_logits=zbuf)
+    _, dw = ops.lmhead_backward(hd, wd, ld, lse, None, gd, need_dhidden=False, dweight=dw_view,
+                                accumulate_dweight=accumulate, saved_logits=zbuf)
+    torch.cuda.synchronize()
+    assert dw.data_ptr() == buf.data_ptr()
+    assert (buf[V * H:] == sentinel).all(), "the weight-gradient GEMM wrote past row V"
+    _, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, g_lp, None, 1.0)
+    assert_close_rel(dw - 0.25 if accumulate else dw, rdw, 1e-2, "dweight")
+
+
+def test_split_k_partials_stay_inside_their_buffer_and_many_ranges_agree(dev):
+    """A dhidden GEMM with few output tiles and a long K (the vocabulary) is cut into many K ranges; the
+    result must equal the oracle, and ragged T (the partial tiles' row count) must not disturb it."""
+    from chatlearn_amd import ops
+    for T, H, V, dtype in ((333, 256, 40000, torch.bfloat16), (130, 64, 30011, torch.float32)):
+        hidden, weight, labels = _inputs(T, H, V, dtype, seed=T, w_std=0.05)
+        g_lp = torch.randn(T, generator=torch.Generator().manual_seed(T + 2))
+        hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+        lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld)
+        dh, dw = ops.lmhead_backward(hd, wd, ld, lse, None, g_lp.to(dev))
+        rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, g_lp, None, 1.0)
+        assert_close_rel(dh, rdh, RTOL[dtype], "dhidden (split K)")
+        assert_rows_rel_l2(dh.float(), rdh, RTOL[dtype], "dhidden rows (split K)")
+        assert_close_rel(dw, rdw, RTOL[dtype], "dweight")
+
+
+def test_kept_logits_beyond_the_half_range_stay_finite(dev):
+    """Kept logits of 16-bit inputs are IEEE half.  A raw logit past the half range (|z| > 65504) is kept as
+    the largest half instead of infinity, so the gradients the backward rebuilds from the kept logits stay
+    finite; every other token's gradient equals the recomputing route's (the saturated token's own
+    probabilities are formed from the saturated value and are not compared)."""
+    from chatlearn_amd import ops
+    T, H, V = 64, 64, 300
+    g = torch.Generator().manual_seed(8)
+    hidden = torch.randn(T, H, generator=g).bfloat16()
+    weight = (torch.randn(V, H, generator=g) * 0.1).bfloat16()
+    hidden[:, 0] = 0.0             # only token 3 reaches the two huge weight entries below
+    hidden[3, :] = 0.0
+    hidden[3, 0] = 300.0
+    weight[7, 0] = 300.0           # z[3, 7] = 90000 > 65504
+    weight[9, 0] = -300.0          # z[3, 9] = -90000
+    labels = torch.randint(0, V, (T,), generator=g)
+    labels[3] = 7
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    g_lp = torch.randn(T, generator=g).to(dev)
+    zbuf = ops.saved_logits_buffer(T, V, torch.bfloat16, dev)
+    lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld, saved_logits=zbuf)
+    z = ops.saved_logits_rowmajor(zbuf, T, V)
+    assert torch.isfinite(z).all()
+    assert float(z[3, 7]) == 65504.0 and float(z[3, 9]) == -65504.0
+    dh, dw = ops.lmhead_backward(hd, wd, ld, lse, None, g_lp, saved_logits=zbuf)
+    assert torch.isfinite(dh.float()).all() and torch.isfinite(dw).all()
+    dh0, dw0 = ops.lmhead_backward(hd, wd, ld, lse, None, g_lp)
+    others = [t for t in range(T) if t != 3]
+    assert_close_rel(dh[others], dh0[others], 2 ** -6, "dhidden of the other tokens, kept against recomputed")
+    # token 3's hidden row is zero outside column 0, so it reaches dW through that column only
+    assert_close_rel(dw[:, 1:], dw0[:, 1:], 2 ** -6, "dweight outside the saturated token's column")

@@ -217,3 +217,36 @@ def test_train_step_entropy_off_means_no_entropy_gradient():
     p_row = [2.0 ** -Q_EXP[(v - 2) % 7] for v in range(7)]
     want_row = [g_lp * ((1.0 if v == 3 else 0.0) - p_row[v]) for v in range(7)]
     assert model.table.grad[2].tolist() == pytest.approx(want_row, rel=1e-6, abs=1e-12)
+
+
+@pytest.mark.parametrize("packing", [False, True])
+def test_train_step_sequence_level_policy(packing):
+    """GSPO on the loop (loss_gallery.py:35-74): every token of a sequence carries the sequence's ratio
+    exp(mean over its masked positions of lp - old); by hand from the RATIO table above
+        s0: masked positions 1,2,3, ratios 1.1, 1.5, 0.5  -> rho0 = (1.1 * 1.5 * 0.5) ** (1/3) = 0.825 ** (1/3)
+        s1: masked positions 0,1,   ratios 0.7, 1.0       -> rho1 = sqrt(0.7)
+        s2: masked position 0,      ratio 1.3             -> rho2 = 1.3
+    clip range [0.8, 1.2]:  s0 (A=+2) unclipped: -2 rho0 per token;  s1 (A=-1): rho1 inside: +rho1 per token;
+    s2 (A=+0.5): max(-0.65, -0.6) = -0.6, clipped, no gradient.  d s_t / d lp_t = 1 (no 1/|y| factor), so the
+    gradient w.r.t. a masked token's logprob of s0 is -2 rho0 / N."""
+    rho0, rho1 = 0.825 ** (1.0 / 3.0), math.sqrt(0.7)
+    pg = (3 * (-2.0 * rho0) + 2 * rho1 - 0.6) / N_RESPONSE_TOKENS
+    model = ToyModel()
+    kw = dict(max_token_in_seq=6) if packing else dict(train_micro_batch_size=3)
+    args = {"entropy_coef": 0.0, "kl_coef": 0.05, "use_group_sequence_policy": True}
+    stats, totals = opl.train_step(model, samples(True), packing=packing, module_args=args, **kw)
+    assert stats["pg_loss"] == pytest.approx(pg, rel=1e-6)
+    assert stats["kl_loss"] == pytest.approx(KL_TOKEN, rel=1e-6)
+    assert float(sum(totals)) == pytest.approx(pg + 0.05 * KL_TOKEN, rel=1e-6)
+    # table row 2 is touched by one masked token only (s0 position 1, label 3), as in the token-level test
+    g_lp = (-2.0 * rho0 + 0.05 * (1.0 - math.exp(-0.1))) / N_RESPONSE_TOKENS
+    p_row = [2.0 ** -Q_EXP[(v - 2) % 7] for v in range(7)]
+    want_row = [g_lp * ((1.0 if v == 3 else 0.0) - p_row[v]) for v in range(7)]
+    assert model.table.grad[2].tolist() == pytest.approx(want_row, rel=1e-6, abs=1e-12)
+    # s2's only masked token (tok 3 -> label 4) is clipped: its row gets the KL gradient only ... tok 3 also sits at
+    # s0 position 2 (masked, label 4, unclipped sequence), so row 3 holds s0's term plus s2's KL term
+    g_s0 = (-2.0 * rho0 + 0.05 * (1.0 - math.exp(-0.1))) / N_RESPONSE_TOKENS
+    g_s2 = (0.05 * (1.0 - math.exp(-0.1))) / N_RESPONSE_TOKENS
+    p_row3 = [2.0 ** -Q_EXP[(v - 3) % 7] for v in range(7)]
+    want_row3 = [(g_s0 + g_s2) * ((1.0 if v == 4 else 0.0) - p_row3[v]) for v in range(7)]
+    assert model.table.grad[3].tolist() == pytest.approx(want_row3, rel=1e-6, abs=1e-12)
