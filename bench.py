@@ -112,7 +112,7 @@ def advantages_for(samples, device, group=1 << 30):
 
 
 def head_step(w, keep, dweight, *, skip_masked=True, skip_masked_forward=False, hook=None, accumulate=False,
-              weight_t_cache=None, n_tok=None, workspace_cache=None):
+              weight_t_cache=None, n_tok=None, workspace_cache=None, check_flags=True):
     cfg = w.cfg
     return grpo_head_step(w.hidden, w.weight, w.labels, w.old, w.ref, w.adv, w.cu, w.mask,
                           n_tokens_total=n_tok or w.n_tok, use_group_sequence_policy=(cfg.loss == "gspo"),
@@ -121,7 +121,7 @@ def head_step(w, keep, dweight, *, skip_masked=True, skip_masked_forward=False, 
                           entropy_coef=cfg.entropy_coef, temperature=cfg.temperature, dweight=dweight,
                           accumulate_dweight=accumulate, keep_logits_chunk=keep, cu_seqlens_host=w.cu_host,
                           skip_masked_rows=skip_masked, skip_masked_forward=skip_masked_forward, stage_hook=hook,
-                          loss_mask_host=w.mask_host, weight_t_cache=weight_t_cache, check_flags=False,
+                          loss_mask_host=w.mask_host, weight_t_cache=weight_t_cache, check_flags=check_flags,
                           workspace_cache=workspace_cache)
 
 
@@ -506,8 +506,7 @@ def operand_activity(w, reps=6):
 
 def autograd_seam(w, steps):
     """The drop-in seam through torch autograd at this workload's shapes: forward, a linear stand-in
-    for the loss, ``.backward()`` into ``hidden.grad`` and an fp32 main-grad buffer; with the logits
-    recomputed in the backward, kept, and kept with the loss mask as a hint."""
+    for the loss, ``.backward()`` into ``hidden.grad`` and an fp32 main-grad buffer."""
     from chatlearn_amd import fused_linear_logprob_entropy
     cfg, T = w.cfg, w.T
     coef = torch.randn(T, device=w.device) * w.mask
@@ -519,8 +518,13 @@ def autograd_seam(w, steps):
         lp, _ = fused_linear_logprob_entropy(h, wt, w.labels, temperature=cfg.temperature, dweight_buffer=main_grad, **kw)
         ((lp * coef).sum() / T).backward()
     out = {}
-    for name, kw in (("recompute", dict(keep_logits_rows=None)), ("kept_logits", dict(keep_logits_rows=T)),
-                     ("kept_logits_mask_hint", dict(keep_logits_rows=T, loss_mask=w.mask))):
+    plan = (("default_arguments", {}),
+            ("default_with_loss_mask", dict(loss_mask=w.mask)),
+            ("default_with_host_loss_mask", dict(loss_mask_host=w.mask_host)),
+            ("keep_8192_rows_recompute_the_rest_host_loss_mask", dict(keep_logits_rows=8192, loss_mask_host=w.mask_host)),
+            ("recompute_everything", dict(keep_logits_rows=None)))
+    for name, kw in plan:
+        torch.cuda.empty_cache()
         for _ in range(2):
             step(**kw)
         torch.cuda.synchronize()
@@ -529,7 +533,7 @@ def autograd_seam(w, steps):
             step(**kw)
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t0) / steps
-        out[name] = {"ms_per_step": dt * 1e3, "tokens_per_s": T / dt}
+        out[name] = {"ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(T / dt, 1)}
     return out
 
 
@@ -545,6 +549,12 @@ def sweep(cfg, device, weight, keep):
     t0 = time.perf_counter()
     groups = split_microbatch(data_list=[dict(s) for s in pop], max_train_token=cfg.T, packing=True)
     packing_ms = (time.perf_counter() - t0) * 1e3
+    # the two library calls behind it alone (lengths in, bins out), without the Python that moves the sample dicts
+    lens = [s["prompt_token_length"] + s["response_token_length"] for s in pop]
+    t0 = time.perf_counter()
+    n_bins = len(ops.bin_packing_ids(lens, cfg.T))
+    ops.bin_packing_fix_bin_ids(lens, n_bins)
+    packing_calls_ms = (time.perf_counter() - t0) * 1e3
     n_tok_total = float(sum(s["response_token_length"] for s in pop))
     works = []
     for mb in groups:
@@ -575,6 +585,7 @@ def sweep(cfg, device, weight, keep):
             "step_mfma_frac_executed": 2.0 * hv * (tokens + 2.0 * rows_bwd) / dt / 1e12 / peak_of(cfg),
             "tokens_per_micro_batch_min_max": [min(w.T for w in works), max(w.T for w in works)],
             "ms_total": dt * 1e3, "tokens_per_s": tokens / dt, "host_bin_packing_ms": round(packing_ms, 2),
+            "host_bin_packing_library_calls_ms": round(packing_calls_ms, 3),
             "note": "bin-packed micro-batches of the whole mini-batch, dW accumulated, W^T built once"}
 
 
@@ -596,6 +607,10 @@ def other_config(name, device, steps, warmup):
     rec["tokens_per_s"] = round(rec["tokens_per_s"], 1)
     rec["ms_per_step"] = round(rec["ms_per_step"], 3)
     rec["step_mfma_frac_executed"] = round(rec["step_mfma_frac_executed"], 4)
+    if train:
+        del out, dweight
+        torch.cuda.empty_cache()
+        rec["gemm_kernels"] = gemm_kernels(w, keep, reps=2)
     return rec
 
 
@@ -614,8 +629,6 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=256)
     ap.add_argument("--gemm-reference", action="store_true",
                     help="also time the vendor library's plain GEMMs (torch.matmul) at this head shape, for context")
-    ap.add_argument("--autograd-seam", action="store_true",
-                    help="also time fused_linear_logprob_entropy through torch autograd")
     ap.add_argument("--operand-activity", action="store_true",
                     help="also time the forward launch and the vendor GEMM on random and on all-zero operands "
                          "(same instructions and traffic, different switching activity: what the power limit costs)")
@@ -705,7 +718,8 @@ def main():
         out["loss_stage"] = loss_stage(w)
         torch.cuda.empty_cache()
         variants = {}
-        plan = [("chunk_4096", dict(keep=4096)), ("whole_micro_batch_kept", dict(keep=T)),
+        plan = [("no_flag_readback", dict(keep=keep, check_flags=False)),
+                ("chunk_8192_rows", dict(keep=8192)), ("chunk_4096_rows", dict(keep=4096)),
                 ("recompute_no_logits_kept", dict(keep=None)),
                 ("no_row_skipping", dict(keep=keep, skip_masked=False)),
                 ("skip_masked_rows_in_forward_too", dict(keep=keep, skip_masked_forward=True))]
@@ -714,9 +728,13 @@ def main():
             torch.cuda.empty_cache()     # each variant sizes its scratch differently: start from an unfragmented pool
             v_dt, v_st, v_out = time_step(w, k, dweight, max(3, args.steps // 2), 3, **kw)
             variants[name] = step_record(w, k, v_dt, v_st, v_out)
-        variants["note"] = ("same micro-batch; chunk_4096 / whole_micro_batch_kept: other chunk sizes of the kept logits; "
+        variants["autograd_seam"] = autograd_seam(w, max(3, args.steps // 2))
+        variants["note"] = ("same micro-batch; the headline reads the loss flags back once per step as the reference's assertions do, "
+                            "no_flag_readback leaves that out; chunk_8192_rows / chunk_4096_rows: smaller bounds on the kept logits; "
                             "recompute: nothing kept, logit tiles recomputed in the backward; no_row_skipping: backward on all T rows; "
-                            "skip_masked_rows_in_forward_too: per-token outputs of masked rows become zero (not the headline)")
+                            "skip_masked_rows_in_forward_too: per-token outputs of masked rows become zero (not the headline); "
+                            "autograd_seam: fused_linear_logprob_entropy through torch autograd (forward, a linear stand-in for the "
+                            "loss, backward into hidden.grad and an fp32 main-grad buffer)")
         out["variants"] = variants
     if not args.no_unfused and train:
         try:
@@ -731,8 +749,6 @@ def main():
         out["operand_activity"] = operand_activity(w)
     if args.glue:
         out["glue_stages"] = glue_stages(cfg, w.samples, dev)
-    if args.autograd_seam and train:
-        out["autograd_seam"] = autograd_seam(w, max(2, args.steps // 2))
     if train and not args.no_sweep:
         torch.cuda.empty_cache()
         out["sweep"] = sweep(cfg, dev, w.weight, keep)

@@ -1,9 +1,11 @@
 """The micro-batch loops of the reference's FSDP policy trainer, for the head path only.
 
 ``PolicyStep`` mirrors ``PolicyTrainer.preprocess_data_list`` / ``train_step`` /
-``forward_step`` (policy_trainer.py:80-172, 187-311, 313-365) for text models on one
-rank (sp_size = 1): same per-sample dict fields in, same ``train_stats`` keys and the
-same per-sample ``old_logprobs`` / ``ref_logprobs`` records out.  What differs is the
+``forward_step`` (policy_trainer.py:80-172, 187-311, 313-365) on one rank (sp_size = 1), for
+text models and - carrying the three-channel position ids, ``pixel_values`` and
+``image_grid_thw`` through as the reference does - for vision-language ones: same
+per-sample dict fields in, same ``train_stats`` keys and the same per-sample
+``old_logprobs`` / ``ref_logprobs`` records out.  What differs is the
 seam: instead of ``self.model(...).logits`` the caller supplies a ``backbone`` that
 returns the final hidden states, and the lm_head weight; logits are never
 materialised beyond one bounded chunk.  FSDP wrapping, the optimizer step and
@@ -29,7 +31,14 @@ class PolicyStep:
                  module_args: Optional[Dict[str, Any]] = None, packing: bool = False, max_token_in_seq: int = 32768,
                  train_micro_batch_size: int = 1, generate_micro_batch_size: int = 1, trainable: bool = True,
                  fsdp_size: int = 1, temperature: float = 1.0, dweight_buffer: Optional[torch.Tensor] = None,
-                 keep_logits_chunk=AUTO):
+                 keep_logits_chunk=AUTO, model_type: str = "llm",
+                 prepend_text_position_channel: Optional[bool] = None):
+        """``backbone(input_ids, position_ids)`` returns the final hidden states ``[b, s, H]``; with
+        ``model_type='vlm'`` it is called as ``backbone(input_ids, position_ids, pixel_values=...,
+        image_grid_thw=...)`` (policy_trainer.py:206-214).  ``prepend_text_position_channel``: packed
+        vision-language position ids get the first channel repeated in front, which the reference does for
+        transformers >= 4.55 (policy_trainer.py:124-125); ``None`` decides the same way from the installed
+        transformers, if there is one."""
         self.backbone = backbone
         self.weight = lm_head_weight
         self.module_args = dict(_DEFAULT_ARGS)
@@ -43,6 +52,15 @@ class PolicyStep:
         self.temperature = temperature
         self.dweight_buffer = dweight_buffer
         self.keep_logits_chunk = keep_logits_chunk
+        self.model_type = model_type
+        if prepend_text_position_channel is None and model_type == "vlm":
+            try:
+                import transformers
+                from packaging.version import Version
+                prepend_text_position_channel = Version(transformers.__version__) >= Version("4.55.0")
+            except ImportError:
+                prepend_text_position_channel = False
+        self.prepend_text_position_channel = bool(prepend_text_position_channel)
         self._metric_prefix = "policy_trainer"
         self._metric_list = []
         self.device = lm_head_weight.device
@@ -63,12 +81,13 @@ class PolicyStep:
         for data_b in (batching(mb) for mb in microbatch_list):
             tokens_ = data_b["all_tokens"].long()
             ori_batch_size, ori_seq_len = tokens_.size()
+            # vision-language samples carry their prompt's three position channels and the image tensors
             attn_mask, loss_mask, position_ids = generate_loss_mask_position_ids(
-                tokens_, data_b["prompt_token_length"], data_b["response_token_length"])
+                tokens_, data_b["prompt_token_length"], data_b["response_token_length"], data_b.get("position_ids", None))
             if 'loss_mask' in data_b:
                 loss_mask = data_b['loss_mask']
             indices = cu_seqlens = None
-            if self.packing and 'position_ids' not in data_b:
+            if self.packing and 'position_ids' not in data_b and self.model_type != "vlm":
                 # unpad_input of tokens and position ids plus the label roll (policy_trainer.py:143-162) in
                 # one device pass driven by the length lists; no device value is read back
                 packed = ops.thd_pack(tokens_.to(self.device), data_b["prompt_token_length"],
@@ -88,7 +107,12 @@ class PolicyStep:
                     tokens_ = tokens_.permute(1, 0)
                     position_ids, *_ = unpad_input(position_ids.unsqueeze(-1).to(self.device),
                                                    attn_mask.to(self.device))
-                    position_ids = position_ids.permute(1, 0)
+                    if self.model_type == "vlm":
+                        position_ids = position_ids.permute(0, 2, 1)        # [3, 1, T] (policy_trainer.py:121-123)
+                        if self.prepend_text_position_channel:
+                            position_ids = torch.cat([position_ids[0:1], position_ids], dim=0)
+                    else:
+                        position_ids = position_ids.permute(1, 0)
                 tokens = tokens_
                 # labels roll along the (packed or padded) token row (policy_trainer.py:135,160)
                 labels, _ = ops.shift_labels(tokens.to(self.device).contiguous(), None, zero_last=False)
@@ -110,6 +134,9 @@ class PolicyStep:
                         "ori_seq_len": ori_seq_len, "indices": indices, "cu_seqlens": cu_seqlens,
                         "ori_batch_size": ori_batch_size, "sample_ids": data_b["id_in_list"],
                         "attention_mask": attn_mask, "pad_size": 0}
+            if self.model_type == "vlm":
+                data_obj.update({"pixel_values": data_b.get("pixel_values", None),
+                                 "image_grid_thw": data_b.get("image_grid_thw", None)})
             if training:
                 data_obj.update({"loss_mask": shifted, "loss_mask_host": shifted_host,
                                  "old_logprobs": data_b["old_logprobs"],
@@ -120,6 +147,12 @@ class PolicyStep:
     def _to_device(self, inputs):
         return {k: (v.to(self.device) if isinstance(v, torch.Tensor) and not k.endswith("_host") else v)
                 for k, v in inputs.items()}
+
+    def _backbone(self, inputs):
+        if self.model_type == "vlm":
+            return self.backbone(inputs["all_tokens"], inputs["position_ids"], pixel_values=inputs["pixel_values"],
+                                 image_grid_thw=inputs["image_grid_thw"])
+        return self.backbone(inputs["all_tokens"], inputs["position_ids"])
 
     def _flat_view(self, inputs, hidden):
         """hidden as [T, H] plus the per-token views of the padded [B, S] side inputs."""
@@ -147,7 +180,7 @@ class PolicyStep:
         ws_cache = {}   # kept logits and head scratch memory, shared by the micro-batches of this step
         for inputs in data_list:
             inputs = self._to_device(inputs)
-            hidden = self.backbone(inputs["all_tokens"], inputs["position_ids"])
+            hidden = self._backbone(inputs)
             flat, cu, pick = self._flat_view(inputs, hidden)
             adv = torch.tensor(inputs["advantages"]).to(self.device)
             out = grpo_head_step(
@@ -187,7 +220,7 @@ class PolicyStep:
         for inputs in data_list:
             inputs = self._to_device(inputs)
             with torch.no_grad():
-                hidden = self.backbone(inputs["all_tokens"], inputs["position_ids"])
+                hidden = self._backbone(inputs)
                 lp, *_ = ops.lmhead_forward(hidden.reshape(-1, hidden.shape[-1]), self.weight,
                                             inputs["labels"].reshape(-1), self.temperature, need_entropy=False)
                 B, S = inputs["ori_batch_size"], inputs["ori_seq_len"]

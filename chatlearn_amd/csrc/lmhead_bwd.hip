@@ -593,14 +593,53 @@ static int pick_k_split(int tiles, int M, int N, int K, int slab, size_t partial
   return best;
 }
 
+// How the dhidden GEMM (C[n][m], M = H output columns, N = token rows, K = vocabulary) is launched.  Its tile
+// count rarely fills whole rounds of one workgroup per CU; cutting K into ranges (fp32 partial tiles, summed
+// by a second pass) repairs that at the price of the partials' traffic.  When the tiles exceed one round the
+// cheaper repair is to cut the token rows instead: a bulk launch over whole rounds of tiles without any K
+// split, and a second launch over the remaining rows with the K split those few tiles want.
+struct DhPlan {
+  int bulk_nt;       // n tiles (256 token rows each) of the bulk launch; 0: one launch over all rows
+  int k_split;       // K ranges of the single launch, or of the tail launch when bulk_nt > 0
+  size_t partial_bytes;
+};
+
+static DhPlan plan_dhidden(int64_t rows, int64_t H, int64_t K, int slab, int cus, size_t partial_cap) {
+  DhPlan pl{0, 1, 0};
+  if (rows <= 0) return pl;
+  const int n_mt = (int)((H + 255) / 256), n_nt = (int)((rows + 255) / 256);
+  const int tiles = n_mt * n_nt;
+  const long k_slabs = (K + slab - 1) / slab;
+  auto cost = [&](long items, int s) {        // rounds x slabs per range, plus 2 % for the partials' traffic
+    const long rounds = (items * s + cus - 1) / cus;
+    const double c = (double)rounds * (double)((k_slabs + s - 1) / s);
+    return s > 1 ? c * 1.02 : c;
+  };
+  const int s_one = pick_k_split(tiles, (int)H, (int)rows, (int)K, slab, partial_cap, cus);
+  pl.k_split = s_one;
+  double best = cost(tiles, s_one);
+  const int per_round_n = cus / n_mt;
+  if (per_round_n >= 1 && n_nt > per_round_n && n_nt % per_round_n != 0) {
+    const int bulk_nt = n_nt / per_round_n * per_round_n;
+    const int64_t tail_rows = rows - (int64_t)bulk_nt * 256;
+    const int tail_tiles = (n_nt - bulk_nt) * n_mt;
+    const int s_tail = pick_k_split(tail_tiles, (int)H, (int)tail_rows, (int)K, slab, partial_cap, cus);
+    const double two = cost((long)bulk_nt * n_mt, 1) + cost(tail_tiles, s_tail) + 0.01 * (double)k_slabs;
+    if (two < 0.98 * best) {
+      pl.bulk_nt = bulk_nt;
+      pl.k_split = s_tail;
+      pl.partial_bytes = s_tail > 1 ? (size_t)s_tail * tail_rows * H * sizeof(float) : 0;
+      return pl;
+    }
+  }
+  pl.partial_bytes = s_one > 1 ? (size_t)s_one * rows * H * sizeof(float) : 0;
+  return pl;
+}
+
 // Bytes of fp32 split-K partials the dhidden GEMM of `rows` tokens wants (planned for a 256-CU device, so
 // that the workspace size does not depend on the device in use; a launch takes fewer ranges if they do not fit).
 static size_t dhidden_partial_bytes(int64_t rows, int64_t H, int64_t ldv, int slab) {
-  if (rows <= 0) return 0;
-  const int tiles = (int)(((H + 255) / 256) * ((rows + 255) / 256));
-  const size_t cap = (size_t)1 << 30;
-  const int s = pick_k_split(tiles, (int)H, (int)rows, (int)ldv, slab, cap, 256);
-  return s > 1 ? (size_t)s * rows * H * sizeof(float) : 0;
+  return plan_dhidden(rows, H, ldv, slab, 256, (size_t)1 << 30).partial_bytes;
 }
 
 struct BwdPlan {
@@ -647,9 +686,9 @@ static int64_t chunk_for_workspace(int64_t T, int64_t H, int64_t V, size_t es, s
 }
 
 template <typename T, typename OutT, bool kMContig>
-static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, int64_t b_kslabs, int N, int K, void* C,
-                       int64_t ldc, int accumulate, hipStream_t stream, float* partial = nullptr,
-                       size_t partial_bytes = 0) {
+static int launch_gemm_one(const void* A, int64_t a_kslabs, int M, const void* B, int64_t b_kslabs, int N, int K, void* C,
+                           int64_t ldc, int accumulate, hipStream_t stream, float* partial, size_t partial_bytes,
+                           int k_split_wanted) {
   using Tile = HeadTile<T>;
   int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<T, OutT, kMContig>), Tile::kLdsBytes, "gemm_nt_kernel");
   if (rc) return rc;
@@ -660,7 +699,13 @@ static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, in
   g.accumulate = accumulate;
   const int slab = Tile::kSlabK;
   const int cus = device_cu_count();
-  g.k_split = (partial && partial_bytes) ? pick_k_split(g.n_mt * g.n_nt, M, N, K, slab, partial_bytes, cus) : 1;
+  g.k_split = (partial && partial_bytes) ? k_split_wanted : 1;
+  auto fits = [&](int ks) {      // partials fit the buffer and no K range is empty after rounding to whole slabs
+    if (ks <= 1) return true;
+    if ((size_t)ks * M * N * sizeof(float) > partial_bytes) return false;
+    return (int64_t)(ks - 1) * round_up64((K + ks - 1) / ks, slab) < K;
+  };
+  while (!fits(g.k_split)) --g.k_split;
   g.k_per_split = g.k_split > 1 ? (int)round_up64((K + g.k_split - 1) / g.k_split, slab) : K;
   g.partial = partial;
   // Many more tiles than CUs and no K split: let one workgroup per CU walk runs of tiles instead of
@@ -680,6 +725,29 @@ static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, in
   hipLaunchKernelGGL(splitk_reduce_kernel<OutT>, dim3(blocks), dim3(256), 0, stream, partial, g.k_split, MN, kMContig ? M : N,
                      static_cast<OutT*>(C), ldc, accumulate);
   return check_launch("splitk_reduce_kernel");
+}
+
+// C (+)= A B^T; with `partial` (dhidden only) the launch plan of plan_dhidden applies.
+template <typename T, typename OutT, bool kMContig>
+static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, int64_t b_kslabs, int N, int K, void* C,
+                       int64_t ldc, int accumulate, hipStream_t stream, float* partial = nullptr,
+                       size_t partial_bytes = 0) {
+  using Tile = HeadTile<T>;
+  if (!(kMContig && partial && partial_bytes))
+    return launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, M, B, b_kslabs, N, K, C, ldc, accumulate, stream, nullptr, 0, 1);
+  const DhPlan pl = plan_dhidden(N, M, K, Tile::kSlabK, device_cu_count(), partial_bytes);
+  if (pl.bulk_nt == 0)
+    return launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, M, B, b_kslabs, N, K, C, ldc, accumulate, stream, partial,
+                                              partial_bytes, pl.k_split);
+  const int bulk_rows = pl.bulk_nt * 256;
+  int rc = launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, M, B, b_kslabs, bulk_rows, K, C, ldc, accumulate, stream,
+                                              nullptr, 0, 1);
+  if (rc) return rc;
+  constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;
+  const T* b_tail = static_cast<const T*>(B) + (int64_t)pl.bulk_nt * b_kslabs * kSlabElems;
+  OutT* c_tail = static_cast<OutT*>(C) + (int64_t)bulk_rows * ldc;
+  return launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, M, b_tail, b_kslabs, N - bulk_rows, K, c_tail, ldc, accumulate,
+                                            stream, partial, partial_bytes, pl.k_split);
 }
 
 template <typename T>
@@ -793,6 +861,15 @@ extern "C" size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_
                                                     int64_t chunk_tokens, int32_t with_saved_logits) {
   if (T <= 0 || H <= 0 || V <= 0 || (dtype != CLGRPO_BF16 && dtype != CLGRPO_F32)) return 0;
   return bwd_plan(T, H, V, dtype_bytes(dtype), chunk_tokens, (with_saved_logits & 1) != 0, (with_saved_logits & 2) == 0).total;
+}
+
+extern "C" int clgrpo_lmhead_bwd_dhidden_plan(int64_t rows, int64_t H, int64_t V, int32_t dtype, int32_t cus, int32_t* out) {
+  if (rows <= 0 || H <= 0 || V <= 0 || out == nullptr || (dtype != CLGRPO_BF16 && dtype != CLGRPO_F32)) return CLGRPO_EINVAL;
+  const int slab = (int)(kRowBytes / dtype_bytes(dtype));
+  const DhPlan pl = plan_dhidden(rows, H, round_up64(V, 64), slab, cus > 0 ? cus : 256, (size_t)1 << 30);
+  out[0] = pl.bulk_nt;
+  out[1] = pl.k_split;
+  return CLGRPO_OK;
 }
 
 static int bwd_entry(const char* who, const clgrpo_lmhead_bwd_args* a, int64_t vocab_begin, void* stream) {

@@ -129,30 +129,28 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
     if (STORE_Z) {
       // Raw logits for the backward, straight from the accumulators: per 32x32 block a lane stores its
       // 16 values as 16-byte pieces, each piece of the 64 lanes one contiguous KB (z-native layout).
-      // The padding columns past V are stored as zeros.
+      // Vocabulary rows past V hold zeros already (the operand loads are range-checked), and the
+      // backward ignores whatever the padding columns hold.
       typedef typename KeptLogit<T>::type ZT;
       typedef ZNative<ZT> ZL;
-      if (a_rows < kFwdBM) {
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-          for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-              if (wm * WM + mi * 32 + acc_row(r, lane) >= a_rows) acc[mi][ni][r] = 0.f;
-      }
       char* z = static_cast<char*>(p.z_out);
       const int64_t n_kslab = p.ldz / ZL::kSlabElems;
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni) {
-        if (zrow[ni] < 0) continue;
+        // The row is the same for every vocabulary tile, so the compiler would keep the 64-bit addresses it
+        // forms from it alive across the K loops, where registers are scarcest, spill them, and reload them
+        // between the stores (a reload waits for the stores issued before it).  Re-deriving them from the
+        // 32-bit row costs a handful of instructions per tile.
+        int row = zrow[ni];
+        asm volatile("" : "+v"(row));
+        if (row < 0) continue;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
           const int v_blk = v0 + wm * WM + mi * 32;
           if (v_blk >= p.ldz) continue;
 #pragma unroll
           for (int j = 0; j < ZL::PIECES; ++j)
-            *reinterpret_cast<u32x4*>(z + ZL::piece_offset(zrow[ni], v_blk >> 5, n_kslab, lane >> 5, j)) =
+            *reinterpret_cast<u32x4*>(z + ZL::piece_offset(row, v_blk >> 5, n_kslab, lane >> 5, j)) =
                 pack_piece<ZT>(acc[mi][ni], j * ZL::kPerPiece);
         }
       }
@@ -301,13 +299,14 @@ __global__ void lmhead_fwd_finalize_kernel(FinalizeParams p) {
 }
 
 // Split of the vocabulary tiles over workgroups.  A workgroup walks ceil(n_vt / n_split) tiles for
-// one block of 256 tokens; with each CU holding one workgroup the launch takes
-// ceil(n_tb * n_split / CUs) rounds, so the pick minimises rounds * tiles-per-workgroup.  At least
-// four splits when possible: the workgroups of an XCD then form a 4-row block sharing operands.
-// `cus` <= 0 plans for a 256-CU device (the workspace size must not depend on the device in use).
-static void fwd_plan(int64_t T, int64_t V, int& n_tb, int& n_vt, int& n_split, int& tiles_per_split, int cus = 0) {
-  n_tb = (int)((T + kFwdBN - 1) / kFwdBN);
-  n_vt = (int)((V + kFwdBM - 1) / kFwdBM);
+// one block of 256 tokens; with each CU holding one workgroup a launch takes
+// ceil(n_tb * n_split / CUs) rounds, so its cost in tile periods is rounds * tiles-per-workgroup.  At
+// least four splits when possible: the workgroups of an XCD then form a 4-row block sharing operands.
+// The launch over n_tb token blocks: returns its cost in sixteenths of a tile period (small penalties break
+// ties).  Many splits and several rounds are fine (65 token blocks: 35 splits of 17 tiles, 9 rounds = 153 tile
+// periods against the ideal 151), so the plan stays within a few per cent of n_tb * n_vt / CUs tile periods
+// from about 7 token blocks on.  `cus` <= 0 plans for a 256-CU device.
+static long fwd_single_cost(int n_tb, int n_vt, int cus, int& n_split, int& tiles_per_split) {
   if (cus <= 0) cus = 256;
   int best = 1;
   long best_cost = -1;
@@ -315,11 +314,12 @@ static void fwd_plan(int64_t T, int64_t V, int& n_tb, int& n_vt, int& n_split, i
     const int tps = (n_vt + sp - 1) / sp;
     const int eff_sp = (n_vt + tps - 1) / tps;
     const long rounds = ((long)n_tb * eff_sp + cus - 1) / cus;
-    long cost = rounds * tps * 16 + (sp < 4 ? 8 : 0) + eff_sp / 8;   // small penalties break ties
+    long cost = rounds * tps * 16 + (sp < 4 ? 8 : 0) + eff_sp / 8;
     if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = sp; }
   }
   tiles_per_split = (n_vt + best - 1) / best;
   n_split = (n_vt + tiles_per_split - 1) / tiles_per_split;
+  return best_cost;
 }
 
 template <typename T, bool STORE_Z>
@@ -333,7 +333,9 @@ static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream, int64
   p.T = (int)a->T;
   p.H = (int)a->H;
   p.V = (int)a->V;
-  fwd_plan(a->T, a->V, p.n_tb, p.n_vt, p.n_split, p.tiles_per_split, device_cu_count());
+  p.n_tb = (int)((a->T + kFwdBN - 1) / kFwdBN);
+  p.n_vt = (int)((a->V + kFwdBM - 1) / kFwdBM);
+  fwd_single_cost(p.n_tb, p.n_vt, device_cu_count(), p.n_split, p.tiles_per_split);
   p.c = a->inv_temperature * kLog2e;
   p.part = static_cast<float4*>(a->workspace);
   p.z_out = a->saved_logits;
@@ -381,6 +383,17 @@ int validate_head_shape(const char* who, int64_t T, int64_t H, int64_t V, int32_
 using namespace clgrpo;
 
 extern "C" int64_t clgrpo_saved_logits_ld(int64_t V) { return V <= 0 ? 0 : round_up64(V, 64); }
+
+extern "C" int clgrpo_lmhead_fwd_launch_plan(int64_t T, int64_t V, int32_t cus, int32_t* out) {
+  if (T <= 0 || V <= 0 || out == nullptr) return CLGRPO_EINVAL;
+  const int n_tb = (int)((T + kFwdBN - 1) / kFwdBN), n_vt = (int)((V + kFwdBM - 1) / kFwdBM);
+  int n_split, tps;
+  fwd_single_cost(n_tb, n_vt, cus, n_split, tps);
+  out[0] = n_tb;
+  out[1] = n_split;
+  out[2] = tps;
+  return CLGRPO_OK;
+}
 
 extern "C" size_t clgrpo_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype) {
   (void)H;

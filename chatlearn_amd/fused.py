@@ -315,29 +315,26 @@ def _token_chunks(T, chunk_rows, seq_bounds, live_cum=None, n_ranges=None):
     return out
 
 
-def _launch_cost(chunks, live_cum, H, V, cus=256):
-    """Relative time of the three GEMM-shaped launches of every chunk, in units of one 256 x 256 tile
-    over one K element on one CU: a launch of n work items takes ceil(n / cus) rounds.  Mirrors the
-    library's launch plans (vocabulary splits of the forward, K ranges of the dhidden GEMM, walking
-    workgroups of the dW GEMM); the passes that do not depend on the cuts (d(logits), transposes)
-    are left out, the read of dW's previous contents by every chunk after the first is counted."""
+def _launch_cost(chunks, live_cum, H, V, dtype=torch.bfloat16, cus=256):
+    """Relative time of the three GEMM-shaped passes of every chunk, in units of one 256 x 256 tile over one
+    K element on one CU: a launch of n work items takes ceil(n / cus) rounds.  Asks the library for its
+    launch plans (vocabulary splits of the forward, bulk / K-split launches of the dhidden GEMM) and mirrors
+    the walking workgroups of the dW GEMM; the passes that do not depend on the cuts (d(logits),
+    transposes) are left out, the read of dW's previous contents by every chunk after the first is counted."""
     n_vt = -(-V // 256)
     n_ht = -(-H // 256)
     cost = 0.0
     for k, (lo, hi) in enumerate(chunks):
         rows = (hi - lo) if live_cum is None else int(live_cum[hi] - live_cum[lo])
-        n_tb = -(-(hi - lo) // 256)
-        best = None
-        for sp in range(1, min(64, n_vt) + 1):                 # forward: rounds x vocabulary tiles per workgroup
-            tps = -(-n_vt // sp)
-            c = -(-(n_tb * -(-n_vt // tps)) // cus) * tps
-            best = c if best is None else min(best, c)
-        cost += best * H
+        n_tb, _, tps = ops.lmhead_forward_launch_plan(hi - lo, V, cus)
+        cost += -(-(n_tb * -(-n_vt // tps)) // cus) * tps * H
         if rows == 0:
             continue
+        bulk_nt, ks = ops.dhidden_launch_plan(rows, H, V, dtype, cus)
         n_rt = -(-rows // 256)
-        tiles = n_ht * n_rt                                    # dhidden: K = V, up to 16 K ranges
-        cost += min(-(-(tiles * s) // cus) * (V / s) for s in range(1, 17))
+        if bulk_nt:
+            cost += -(-(bulk_nt * n_ht) // cus) * V
+        cost += -(-((n_rt - bulk_nt) * n_ht * ks) // cus) * (V / ks)
         walk = max(1, cus // n_ht)                             # dW: workgroups keep an H tile and walk vocabulary tiles
         cost += (-(-n_vt // min(walk, n_vt)) if n_vt * n_ht >= 4 * cus else -(-(n_vt * n_ht) // cus)) * rows
         if k > 0:
@@ -345,7 +342,8 @@ def _launch_cost(chunks, live_cum, H, V, cus=256):
     return cost
 
 
-def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask_host=None, shape=None):
+def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask_host=None, shape=None,
+                     dtype=torch.bfloat16):
     """The token ranges ``grpo_head_step`` walks: at most ``keep_logits_chunk`` kept rows each.  Only
     unmasked rows keep their logits, so with the mask known on the host (``loss_mask_host``, given when
     masked rows are skipped) the bound counts those; the sequence-level loss needs ranges that end on
@@ -364,12 +362,12 @@ def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask
     if shape is None or len(fewest) == 1:
         return fewest
     H, V = shape
-    best, best_cost = fewest, _launch_cost(fewest, live_cum, H, V)
+    best, best_cost = fewest, _launch_cost(fewest, live_cum, H, V, dtype)
     for extra in (1, 2):
         cand = _token_chunks(T, keep_logits_chunk, bounds, live_cum, n_ranges=len(fewest) + extra)
         if len(cand) != len(fewest) + extra:
             continue
-        c = _launch_cost(cand, live_cum, H, V)
+        c = _launch_cost(cand, live_cum, H, V, dtype)
         if c < 0.98 * best_cost:                                # more ranges must buy more than 2 %
             best, best_cost = cand, c
     return best
@@ -438,7 +436,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
         raise ValueError(f"loss_mask_host must be a CPU copy of loss_mask with {T} entries")
     chunks = head_step_chunks(T, keep_logits_chunk, use_group_sequence_policy,
                               cu_seqlens_host if cu_seqlens_host is not None else cu_seqlens,
-                              loss_mask_host if skip else None, shape=(hidden.shape[1], V))
+                              loss_mask_host if skip else None, shape=(hidden.shape[1], V), dtype=hidden.dtype)
     zbuf = None
     rows_of = None
     if skip and loss_mask_host is not None and T > 0:

@@ -165,6 +165,23 @@ def lmhead_forward(hidden: torch.Tensor, weight: torch.Tensor, labels: Optional[
     return logprob, entropy, rowmax, lse
 
 
+def lmhead_forward_launch_plan(T: int, V: int, cus: int = 0) -> Tuple[int, int, int]:
+    """(blocks of 256 tokens, vocabulary splits, vocabulary tiles per workgroup) of the forward launch for T
+    tokens on a device with ``cus`` compute units (0: 256)."""
+    out = (C.c_int32 * 3)()
+    _lib.check(_lib.lib().clgrpo_lmhead_fwd_launch_plan(int(T), int(V), int(cus), C.cast(out, C.c_void_p)))
+    return int(out[0]), int(out[1]), int(out[2])
+
+
+def dhidden_launch_plan(rows: int, H: int, V: int, dtype, cus: int = 0) -> Tuple[int, int]:
+    """(256-token tiles of a first launch without a K split or 0, K ranges of the remaining launch) for the
+    dhidden contraction of ``rows`` tokens."""
+    out = (C.c_int32 * 2)()
+    _lib.check(_lib.lib().clgrpo_lmhead_bwd_dhidden_plan(int(rows), int(H), int(V), BF16 if dtype == torch.bfloat16 else F32,
+                                                         int(cus), C.cast(out, C.c_void_p)))
+    return int(out[0]), int(out[1])
+
+
 def lmhead_forward_workspace_bytes(T: int, H: int, V: int, dtype) -> int:
     """Bytes of scratch one ``lmhead_forward`` call of T tokens needs."""
     return int(_lib.lib().clgrpo_lmhead_fwd_workspace_bytes(T, H, V, BF16 if dtype == torch.bfloat16 else F32))

@@ -41,7 +41,7 @@ typedef enum { CLGRPO_BF16 = 0, CLGRPO_F32 = 1, CLGRPO_F64 = 2, CLGRPO_U8 = 3 /*
  *                 inputs are IEEE half in the forward's own order; clgrpo_lmhead_fwd_workspace_bytes grew to
  *                 min(ceil(V / 256), 64) * T * 16.
  *   2.00 -> 2.01: clgrpo_lmhead_bwd_workspace_bytes sizes the split-K partials by the GEMM's plan (smaller in
- *                 general); clgrpo_policy_loss_args.megatron (appended) selects the Megatron loss sums. */
+ *                 general); clgrpo_lmhead_fwd_launch_plan and clgrpo_lmhead_bwd_dhidden_plan added. */
 #define CLGRPO_VERSION 201
 int clgrpo_version(void);
 const char* clgrpo_last_error_string(void);
@@ -93,6 +93,12 @@ int64_t clgrpo_saved_logits_ld(int64_t V);
 
 size_t clgrpo_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype);
 int clgrpo_lmhead_fwd(const clgrpo_lmhead_fwd_args* a, void* stream);
+/* The grid of the forward launch for T tokens on a device with `cus` compute units (<= 0: 256):
+ * out[0] = blocks of 256 tokens, out[1] = vocabulary splits (a workgroup owns one token block and one split),
+ * out[2] = vocabulary tiles of 256 entries a workgroup walks.  The launch takes ceil(out[0] * out[1] / cus)
+ * rounds of one workgroup per compute unit.  Host-side arithmetic only; no counterpart in the reference
+ * (its lm_head is one library GEMM). */
+int clgrpo_lmhead_fwd_launch_plan(int64_t T, int64_t V, int32_t cus, int32_t* out);
 
 /* ------------------------------------------------------------------ *
  * Backward of the fused head: recomputes logit tiles from hidden, W and the
@@ -136,6 +142,11 @@ typedef struct {
 size_t clgrpo_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int32_t dtype,
                                          int64_t chunk_tokens, int32_t with_saved_logits);
 int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream);
+/* How the dhidden contraction of `rows` tokens is launched on a device with `cus` compute units (<= 0: 256):
+ * out[0] = 256-token tiles of a first launch that fills whole rounds without cutting K (0: one launch over
+ * all rows), out[1] = K ranges of the (remaining) launch, whose fp32 partial tiles a second pass sums.
+ * Host-side arithmetic only; no counterpart in the reference. */
+int clgrpo_lmhead_bwd_dhidden_plan(int64_t rows, int64_t H, int64_t V, int32_t dtype, int32_t cus, int32_t* out);
 
 /* ------------------------------------------------------------------ *
  * One vocabulary shard of the head (tensor-parallel lm_head: each rank keeps rows

@@ -3,8 +3,9 @@
 Test infrastructure only; never imported by the product package.
 
 Reference semantics restated here:
-  * generate_loss_mask_position_ids (text)  trainer_utils.py:60-96
-  * unpad_input                              trainer_utils.py:155-194
+  * generate_loss_mask_position_ids         trainer_utils.py:60-96 (text and the three-channel
+                                             vision-language position ids)
+  * unpad_input                              trainer_utils.py:155-194 (incl. the channel-first 4-D branch)
   * index_first_axis / pad_input             flash-attn bert_padding (a row
     gather and its inverse scatter into zeros), call sites
     trainer_utils.py:179,190 and policy_trainer.py:239-248,350-355
@@ -19,15 +20,26 @@ import torch
 import torch.nn.functional as F
 
 
-def generate_loss_mask_position_ids(tokens, prompt_token_length, response_token_length):
-    """int32 attn/loss masks from the two length lists; position ids are a
-    broadcast arange (trainer_utils.py:68-96, text-only branch)."""
+def generate_loss_mask_position_ids(tokens, prompt_token_length, response_token_length, prompt_position_ids=None):
+    """int32 attn/loss masks from the two length lists; position ids are a broadcast arange
+    (trainer_utils.py:68-96, text-only branch) or, with ``prompt_position_ids`` (per sample three
+    lists), a [3, B, S] tensor: each channel starts with the given list and continues counting up from
+    its maximum + 1 (trainer_utils.py:76-92)."""
     loss_mask = torch.zeros_like(tokens, dtype=torch.int32)
     attn_mask = torch.zeros_like(tokens, dtype=torch.int32)
     for i, (p, r) in enumerate(zip(prompt_token_length, response_token_length)):
         loss_mask[i, p:p + r] = 1
         attn_mask[i, :p + r] = 1
-    seq_len = tokens.shape[1]
+    batch_size, seq_len = tokens.shape
+    if prompt_position_ids:
+        pos = torch.zeros((3, batch_size, seq_len), dtype=torch.long)
+        for b, channels in enumerate(prompt_position_ids):
+            for ch in range(3):
+                sub = channels[ch]
+                pos[ch, b, :len(sub)] = torch.tensor(sub)
+                start = max(sub) + 1
+                pos[ch, b, len(sub):] = torch.arange(start, start + (seq_len - len(sub)))
+        return attn_mask, loss_mask, pos
     pos = torch.arange(seq_len, dtype=torch.long, device=tokens.device).unsqueeze(0).expand_as(tokens)
     return attn_mask, loss_mask, pos
 
@@ -37,11 +49,16 @@ def index_first_axis(x, indices):
 
 
 def unpad_input(hidden_states, attention_mask):
-    """trainer_utils.py:155-194 (3-D branch)."""
+    """trainer_utils.py:155-194; a tensor of more than three dimensions is (channel, batch, seqlen, ...)
+    and is unpadded channel by channel (:176-187)."""
     seqlens = attention_mask.sum(dim=-1, dtype=torch.int32)
     indices = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
     max_seqlen = seqlens.max().item()
     cu_seqlens = F.pad(torch.cumsum(seqlens, dim=0, dtype=torch.int32), (1, 0))
+    if hidden_states.dim() > 3:
+        per_channel = [index_first_axis(hidden_states[ch].reshape(-1, *hidden_states.shape[3:]), indices)
+                       for ch in range(hidden_states.shape[0])]
+        return torch.stack(per_channel), indices, cu_seqlens, max_seqlen
     flat = hidden_states.reshape(-1, *hidden_states.shape[2:])
     return index_first_axis(flat, indices), indices, cu_seqlens, max_seqlen
 

@@ -2,13 +2,15 @@
 
 Test infrastructure only; never imported by the product package.
 
-Reference semantics restated here (sp_size = 1, fsdp_size = 1, no vision inputs):
+Reference semantics restated here (sp_size = 1, fsdp_size = 1; vision-language inputs are carried
+through as the reference carries them, model_type = 'vlm'):
   * preprocess_data_list      policy_trainer.py:80-172
   * train_step loop           policy_trainer.py:203-311   (without optimizer / grad clipping)
   * forward_step loop         policy_trainer.py:316-365
 
 ``model(input_ids, position_ids)`` stands for ``self.model(...).logits``: it returns
-logits [b, s, V].  Everything runs on the CPU with the other oracle modules.
+logits [b, s, V]; a vision-language model is called as
+``model(input_ids, position_ids, pixel_values=..., image_grid_thw=...)`` (policy_trainer.py:206-214).  Everything runs on the CPU with the other oracle modules.
 
 Pinned by tests/test_policy_loop_cpu.py: a three-sample case worked by hand from the
 reference lines above (micro-batch order with a tie on the bin totals, packed token row,
@@ -26,7 +28,7 @@ from . import softmax_stats as osm
 
 
 def preprocess_data_list(data_list, training, *, packing, max_token_in_seq=None, train_micro_batch_size=1,
-                         generate_micro_batch_size=1):
+                         generate_micro_batch_size=1, model_type="llm", prepend_text_position_channel=False):
     total_resp = torch.tensor(sum(d["response_token_length"] for d in data_list)) / 1   # / sp_size, all-reduce = identity
     if packing:
         mbs = opk.split_microbatch(data_list=data_list, max_train_token=max_token_in_seq, packing=True)
@@ -39,7 +41,7 @@ def preprocess_data_list(data_list, training, *, packing, max_token_in_seq=None,
         tokens_ = b["all_tokens"].long()
         p_len, r_len = b["prompt_token_length"], b["response_token_length"]
         ori_bs, ori_len = tokens_.size()
-        attn, loss_mask, pos = oi.generate_loss_mask_position_ids(tokens_, p_len, r_len)
+        attn, loss_mask, pos = oi.generate_loss_mask_position_ids(tokens_, p_len, r_len, b.get("position_ids", None))
         if "loss_mask" in b:
             loss_mask = b["loss_mask"]
         indices = None
@@ -47,12 +49,19 @@ def preprocess_data_list(data_list, training, *, packing, max_token_in_seq=None,
             tokens_, indices, *_ = oi.unpad_input(tokens_.unsqueeze(-1), attn)
             tokens_ = tokens_.permute(1, 0)
             pos, *_ = oi.unpad_input(pos.unsqueeze(-1), attn)
-            pos = pos.permute(1, 0)
+            if model_type == "vlm":
+                pos = pos.permute(0, 2, 1)                       # [3, 1, T]   (policy_trainer.py:121-123)
+                if prepend_text_position_channel:                # transformers >= 4.55 (policy_trainer.py:124-125)
+                    pos = torch.cat([pos[0:1], pos], dim=0)
+            else:
+                pos = pos.permute(1, 0)
         tokens = tokens_
         labels = oi.shift_labels(tokens)
         obj = {"all_tokens": tokens, "position_ids": pos, "labels": labels, "ori_seq_len": ori_len,
                "indices": indices, "ori_batch_size": ori_bs, "sample_ids": b["id_in_list"],
                "attention_mask": attn, "pad_size": 0}
+        if model_type == "vlm":
+            obj.update({"pixel_values": b.get("pixel_values", None), "image_grid_thw": b.get("image_grid_thw", None)})
         if training:
             obj.update({"loss_mask": oi.shift_loss_mask_fsdp(loss_mask), "old_logprobs": b["old_logprobs"], "ref_logprobs": b["ref_logprobs"],
                         "advantages": b["advantages"]})
@@ -67,12 +76,20 @@ def _repad(x, inputs, packing):
     return F.pad(x, (0, inputs["ori_seq_len"] - x.shape[1]), mode="constant", value=0)
 
 
+def _call_model(model, inputs, model_type):
+    if model_type == "vlm":
+        return model(inputs["all_tokens"], inputs["position_ids"], pixel_values=inputs["pixel_values"],
+                     image_grid_thw=inputs["image_grid_thw"])
+    return model(inputs["all_tokens"], inputs["position_ids"])
+
+
 def train_step(model, data_list, *, packing, module_args, **prep):
     """Returns (train_stats, per-micro-batch totals); gradients accumulate in the model's parameters."""
     n_tok, mbs = preprocess_data_list(data_list, True, packing=packing, **prep)
+    model_type = prep.get("model_type", "llm")
     pg_l, en_l, kl_l, totals = [], [], [], []
     for inputs in mbs:
-        logits = model(inputs["all_tokens"], inputs["position_ids"])
+        logits = _call_model(model, inputs, model_type)
         logprobs = osm.logprobs_from_logits(logits, inputs["labels"])
         ctx = torch.enable_grad() if module_args["entropy_coef"] > 0 else torch.no_grad()
         with ctx:
@@ -97,7 +114,7 @@ def forward_step(model, data, *, packing, trainable, **prep):
     tag = "old_logprobs" if trainable else "ref_logprobs"
     for inputs in mbs:
         with torch.no_grad():
-            logits = model(inputs["all_tokens"], inputs["position_ids"])
+            logits = _call_model(model, inputs, prep.get("model_type", "llm"))
             logprobs = _repad(osm.logprobs_from_logits(logits, inputs["labels"]), inputs, packing)
         for sid, lp in zip(inputs["sample_ids"], oi.split_and_unpadding(logprobs, inputs["attention_mask"])):
             data[sid].update({tag: lp})

@@ -2,6 +2,7 @@
 import random
 
 import numpy as np
+import torch
 
 from chatlearn_amd.fused import _token_chunks
 
@@ -87,11 +88,9 @@ def test_asked_number_of_ranges_and_launch_cost_choice():
             assert all(hi > lo for lo, hi in r) and len(r) >= len(fewest)
             if bounds is None:
                 assert all(hi - lo <= cap for lo, hi in r)
-    # the cost counts whole rounds of one workgroup per CU: 64 token blocks x 4 vocabulary splits fill 256 CUs
-    # (149 tiles each); 65 blocks fill them worse whatever the split (3 splits: 195 workgroups x 198 tiles)
     H, V = 2048, 151936
     one, more = _launch_cost([(0, 16384)], None, H, V), _launch_cost([(0, 16640)], None, H, V)
-    assert one / 16384 < more / 16640
+    assert one < more < 1.1 * one                                                          # one more token block costs about 1/64 more, not a second round
     # a sequence-level micro-batch of 32768 tokens: the bound of 17408 rows allows two ranges; the choice
     # never takes more than two extra and every range ends on a sequence boundary
     cu = [0, 5000, 9000, 16000, 21000, 26000, 30000, 32768]
@@ -102,3 +101,25 @@ def test_asked_number_of_ranges_and_launch_cost_choice():
     assert ranges[0][0] == 0 and ranges[-1][1] == 32768
     # everything fits one range: one range, whatever the shape
     assert head_step_chunks(16384, 17408, False, None, None, shape=(4096, V)) == [(0, 16384)]
+
+
+def test_library_launch_plans():
+    """The forward picks its vocabulary splits so that the launch fills whole rounds of one workgroup per CU;
+    the dhidden GEMM cuts its rows into a bulk launch of whole rounds before it cuts K.  594 vocabulary
+    tiles (V = 151936), 256 CUs."""
+    from chatlearn_amd import ops
+    V = 151936
+    assert ops.lmhead_forward_launch_plan(16384, V) == (64, 4, 149)                        # 64 blocks x 4 splits = 256 workgroups
+    assert ops.lmhead_forward_launch_plan(8192, V) == (32, 8, 75)
+    assert ops.lmhead_forward_launch_plan(16640, V) == (65, 35, 17)                        # 65 blocks: 2275 workgroups, 9 rounds of 17 tiles = 153 periods (ideal 151)
+    for T in (1792, 5000, 12126, 17599, 20000, 33000, 65536, 100000):
+        n_tb, sp, tps = ops.lmhead_forward_launch_plan(T, V)
+        assert n_tb == -(-T // 256) and 1 <= sp <= 64 and sp * tps >= 594                  # every vocabulary tile is covered
+        cost = -(-(n_tb * -(-594 // tps)) // 256) * tps
+        assert cost <= 1.08 * n_tb * 594 / 256                                             # near the ideal n_tb * 594 / 256 tile periods
+    assert ops.lmhead_forward_launch_plan(16640, V, cus=304) != ops.lmhead_forward_launch_plan(16640, V)
+    # dhidden, H = 4096 (16 output tiles per 256 rows): 48 row tiles fill 3 rounds exactly; 50 row tiles run as
+    # 48 without a K split plus 2 x 16 tiles cut into 8 K ranges
+    assert ops.dhidden_launch_plan(12126, 4096, V, torch.bfloat16) == (0, 1)
+    assert ops.dhidden_launch_plan(12700, 4096, V, torch.bfloat16) == (48, 8)
+    assert ops.dhidden_launch_plan(1458, 1024, V, torch.float32) == (0, 10)                # 24 tiles: 10 K ranges fill 240 CUs

@@ -14,8 +14,9 @@ pytestmark = pytest.mark.gpu
 
 CFG = synthetic.CONFIGS["c2"]
 # Smallest fraction of bf16 dW entries that must sit inside |err| <= atol + 1e-2 |ref|, atol = 1e-2
-# median|ref| (see tests/test_gpu_head_step.py::DW_FRAC_BF16 for why it is not 1).
-DW_FRAC_BF16 = 0.999
+# median|ref| (see tests/test_gpu_head_step.py::DW_FRAC_BF16 for why it is not 1); measured on the MI355X at the
+# full head shapes: c2 0.999917, c3 0.999986, c5 0.999994.
+DW_FRAC_BF16 = {"c2": 0.9998, "c3": 0.99995, "c5": 0.99997}
 
 
 @pytest.fixture(scope="module")
@@ -260,7 +261,7 @@ def test_full_head_shapes_forward_backward_against_the_float64_oracle(dev, name,
     assert_rows_rel_l2(dh, rdh, 1e-2, f"{name} dhidden rows")
     assert_rows_rel_l2(dw, rdw, 1e-2, f"{name} dweight rows")
     ours_dh = assert_contract(dh, rdh, 1e-2, f"{name} dhidden")
-    ours_dw = assert_contract(dw, rdw, 1e-2, f"{name} dweight", min_frac=DW_FRAC_BF16)
+    ours_dw = assert_contract(dw, rdw, 1e-2, f"{name} dweight", min_frac=DW_FRAC_BF16[name])
     if name == "c2":
         # the reference's own bf16 arithmetic on the same inputs (temperature 1): this path is at least as close
         # to the float64 result as that, output by output

@@ -39,9 +39,12 @@ CASES = [
 # 1e-2 median|ref|).  The rest are entries whose terms cancel to well below the tensor's typical
 # magnitude; their error is the bf16 rounding of d(logits) (2^-9 relative per term, the same rounding the
 # reference's bf16 autograd applies), not a wrong term: the row-wise L2 and max-norm bounds above hold at 1e-2.
-DW_FRAC_BF16 = 0.995
-# fp32: the same cancelling entries against fp32 accumulation order, a few in 10^4.
-DW_FRAC_FP32 = 0.999
+# The bound asserted per case is what the MI355X measures for it less 5e-4 (measured: c2 0.99928, c3 0.99715,
+# c5 0.99559 at these CPU-sized shapes, where a dW entry sums a few thousand tokens; at the full head shapes
+# tests/test_gpu_fullsize.py asserts 0.9998 and more), so that a regression of a few entries in ten thousand fails.
+DW_FRAC_BF16 = {"c2": 0.9988, "c3": 0.9966, "c5": 0.9951}
+# fp32: the same cancelling entries against fp32 accumulation order, a few in 10^4 (measured 0.99956).
+DW_FRAC_FP32 = 0.9991
 
 
 @pytest.mark.parametrize("name,kw", CASES, ids=[c[0] for c in CASES])
@@ -81,7 +84,7 @@ def test_head_step_matches_oracle(dev, name, kw, keep):
     assert_rows_rel_l2(got["dhidden"].float(), want["dhidden"], rt, "dhidden rows")
     assert_rows_rel_l2(got["dweight"], want["dweight"], rt, "dweight rows")
     assert_contract(got["dhidden"], want["dhidden"], rt, "dhidden")
-    assert_contract(got["dweight"], want["dweight"], rt, "dweight", min_frac=DW_FRAC_FP32 if fp32 else DW_FRAC_BF16)
+    assert_contract(got["dweight"], want["dweight"], rt, "dweight", min_frac=DW_FRAC_FP32 if fp32 else DW_FRAC_BF16[name])
     if keep is not None:
         # masked-out rows were left out of the backward: exact zeros there, and fewer rows projected
         assert got["rows_projected_bwd"] == int(mask.sum())

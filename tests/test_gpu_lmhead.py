@@ -74,8 +74,9 @@ def test_backward_matches_oracle(dev, T, H, V, dtype, temp, with_entropy):
     if dtype == torch.float32:
         assert_contract(dh, rdh, r, "dhidden")
         # dW entries are sums over all tokens; where the terms cancel to far below the tensor's typical
-        # magnitude, fp32 accumulation (any order) is further than 1e-5 from the float64 sum: a few in 10^4
-        assert_contract(dw, rdw, r, "dweight", min_frac=0.999)
+        # magnitude, fp32 accumulation (any order) is further than 1e-5 from the float64 sum: at most 4 entries in
+        # 10^5 on the MI355X
+        assert_contract(dw, rdw, r, "dweight", min_frac=0.9999)
 
 
 def test_backward_chunked_equals_unchunked_and_accumulates(dev):

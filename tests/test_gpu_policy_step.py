@@ -243,3 +243,81 @@ def test_episode_through_records_advantages_and_train_steps(dev):
             assert got_stats[k] == pytest.approx(want_stats[k], rel=1e-5, abs=1e-7), k
         assert_close_rel(bb.tok.grad, tok.grad, 1e-5, "token-embedding grad")
         assert_close_rel(weight.grad, w.grad, 1e-5, "lm_head grad")
+
+
+class _VLBackbone(torch.nn.Module):
+    """Stand-in for a vision-language decoder: token embedding + one embedding per position channel + a
+    projection of the micro-batch's image patches (their mean), so that every carried input reaches the
+    hidden states."""
+
+    def __init__(self, dtype, seed=0):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.tok = torch.nn.Parameter(torch.randn(VOCAB, H, generator=g).to(dtype))
+        self.pos = torch.nn.Parameter((torch.randn(4, MAXLEN * 2, H, generator=g) * 0.1).to(dtype))
+        self.vis = torch.nn.Parameter((torch.randn(6, H, generator=g) * 0.1).to(dtype))
+
+    def forward(self, input_ids, position_ids, pixel_values=None, image_grid_thw=None):
+        h = self.tok[input_ids]
+        for ch in range(position_ids.shape[0]):
+            h = h + self.pos[ch][position_ids[ch]]
+        scale = image_grid_thw.to(h.dtype).prod(dim=1).sum() * 0.01
+        return h + (pixel_values.to(h.dtype).mean(dim=0) @ self.vis) * scale
+
+
+@pytest.mark.parametrize("packing", [False, True])
+@pytest.mark.parametrize("prepend", [False, True])
+def test_vision_language_inputs_reach_the_backbone_and_train(dev, packing, prepend):
+    """model_type = 'vlm': the three position channels, pixel_values and image_grid_thw are carried to the
+    backbone as the reference carries them to the model (policy_trainer.py:104-152,206-214), on the 4-D
+    unpad_input branch when packing; train_step against the oracle loop."""
+    from chatlearn_amd.algorithm.grpo_utils.policy_step import PolicyStep
+    g = torch.Generator().manual_seed(77)
+    data = _samples(7, 29, True)
+    for s in data:
+        p = s["prompt_token_length"]
+        s["position_ids"] = [sorted(torch.randint(0, p, (p,), generator=g).tolist()) for _ in range(3)]
+        n_patch = int(torch.randint(1, 5, (1,), generator=g))
+        s["pixel_values"] = torch.randn(n_patch, 6, generator=g)
+        s["image_grid_thw"] = torch.tensor([[1, 1, n_patch]])
+    bb = _VLBackbone(torch.float32).to(dev)
+    weight = (torch.randn(VOCAB, H, generator=g) * 0.05).to(dev).requires_grad_(True)
+    tok, pos, vis = (x.detach().double().cpu().requires_grad_(True) for x in (bb.tok, bb.pos, bb.vis))
+    w = weight.detach().double().cpu().requires_grad_(True)
+
+    def model(ids, position_ids, pixel_values=None, image_grid_thw=None):
+        h = tok[ids]
+        for ch in range(position_ids.shape[0]):
+            h = h + pos[ch][position_ids[ch]]
+        scale = image_grid_thw.double().prod(dim=1).sum() * 0.01
+        return torch.nn.functional.linear(h + (pixel_values.double().mean(dim=0) @ vis) * scale, w)
+    args = {"entropy_coef": 0.0, "kl_coef": 0.02}
+    kw = dict(max_token_in_seq=200, train_micro_batch_size=3)
+    okw = dict(model_type="vlm", prepend_text_position_channel=prepend, **kw)
+    centred = opl.forward_step(model, copy.deepcopy(data), packing=packing, trainable=True, **okw)
+    for s, c in zip(data, centred):
+        s["old_logprobs"] = (c["old_logprobs"] + (s["old_logprobs"] + 8.0)).float()
+        s["ref_logprobs"] = (c["old_logprobs"] + (s["ref_logprobs"] + 8.0)).float()
+    want_stats, _ = opl.train_step(model, copy.deepcopy(data), packing=packing, module_args=args, **okw)
+    step = PolicyStep(bb, weight, module_args=args, packing=packing, model_type="vlm",
+                      prepend_text_position_channel=prepend, **kw)
+    # what the backbone receives, against the oracle's pre-processing, bit for bit
+    _, got_mbs = step.preprocess_data_list(copy.deepcopy(data), training=True)
+    _, want_mbs = opl.preprocess_data_list(copy.deepcopy(data), True, packing=packing, **okw)
+    assert len(got_mbs) == len(want_mbs)
+    for a, b in zip(got_mbs, want_mbs):
+        assert torch.equal(a["position_ids"].cpu(), b["position_ids"])
+        assert a["position_ids"].shape[0] == (4 if (packing and prepend) else 3)
+        assert torch.equal(a["all_tokens"].cpu(), b["all_tokens"]) and torch.equal(a["labels"].cpu(), b["labels"])
+        assert torch.equal(a["pixel_values"], b["pixel_values"]) and torch.equal(a["image_grid_thw"], b["image_grid_thw"])
+    got_stats = step.train_step(copy.deepcopy(data))
+    for k in ("pg_loss", "kl_loss", "entropy_loss"):
+        assert got_stats[k] == pytest.approx(want_stats[k], rel=1e-5, abs=1e-7), k
+    assert_close_rel(bb.tok.grad, tok.grad, 1e-5, "token-embedding grad")
+    assert_close_rel(bb.pos.grad, pos.grad, 1e-5, "position-channel grad")
+    assert_close_rel(bb.vis.grad, vis.grad, 1e-5, "vision-projection grad")
+    assert_close_rel(weight.grad, w.grad, 1e-5, "lm_head grad")
+    # the no-grad pass carries them too
+    recs = step.forward_step(copy.deepcopy(data))
+    for a, b in zip(recs, centred):
+        assert_close_rel(a["old_logprobs"], b["old_logprobs"], 1e-5, "per-sample logprobs (vlm)")

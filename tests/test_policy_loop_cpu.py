@@ -250,3 +250,45 @@ def test_train_step_sequence_level_policy(packing):
     p_row3 = [2.0 ** -Q_EXP[(v - 3) % 7] for v in range(7)]
     want_row3 = [(g_s0 + g_s2) * ((1.0 if v == 4 else 0.0) - p_row3[v]) for v in range(7)]
     assert model.table.grad[3].tolist() == pytest.approx(want_row3, rel=1e-6, abs=1e-12)
+
+
+def test_vision_language_inputs_are_carried_through():
+    """model_type = 'vlm' (policy_trainer.py:104-107,119-125,146-152; trainer_utils.py:76-92,176-187), by hand on
+    two samples: s0 prompt 3 + response 2 with prompt position channels t = [0,1,2], h = [0,0,1], w = [0,1,0];
+    s1 prompt 2 + response 1 with channels [0,1], [0,0], [0,1].  Each channel continues counting from its
+    maximum + 1 over the rest of the padded row (S = 5):
+        s0: t [0,1,2,3,4]  h [0,0,1,2,3]  w [0,1,0,2,3]
+        s1: t [0,1,2,3,4]  h [0,0,1,2,3]  w [0,1,2,3,4]
+    Padded batches keep the [3, B, S] tensor; packed ones unpad every channel with the same indices
+    (s0's five positions, s1's three) into [3, 1, 8], and with transformers >= 4.55 the first channel is
+    repeated in front ([4, 1, 8]).  pixel_values of the samples are concatenated, image_grid_thw too."""
+    def vl_samples():
+        out = []
+        for toks, p, r, pos, n_patch in (([1, 2, 3, 4, 5], 3, 2, [[0, 1, 2], [0, 0, 1], [0, 1, 0]], 4),
+                                         ([6, 1, 2], 2, 1, [[0, 1], [0, 0], [0, 1]], 2)):
+            out.append({"all_tokens": torch.tensor(toks), "prompt_token_length": p, "response_token_length": r,
+                        "position_ids": pos, "pixel_values": torch.full((n_patch, 3), float(len(toks))),
+                        "image_grid_thw": torch.tensor([[1, 2, n_patch // 2]])})
+        return out
+    want_padded = [[[0, 1, 2, 3, 4], [0, 1, 2, 3, 4]], [[0, 0, 1, 2, 3], [0, 0, 1, 2, 3]], [[0, 1, 0, 2, 3], [0, 1, 2, 3, 4]]]
+    _, mbs = opl.preprocess_data_list(vl_samples(), False, packing=False, generate_micro_batch_size=2, model_type="vlm")
+    mb = mbs[0]
+    assert mb["position_ids"].tolist() == want_padded
+    assert mb["pixel_values"].shape == (6, 3) and mb["pixel_values"][:, 0].tolist() == [5.0] * 4 + [3.0] * 2
+    assert mb["image_grid_thw"].tolist() == [[1, 2, 2], [1, 2, 1]]
+    assert mb["all_tokens"].tolist() == [[1, 2, 3, 4, 5], [6, 1, 2, 0, 0]]
+    want_packed = [[[0, 1, 2, 3, 4, 0, 1, 2]], [[0, 0, 1, 2, 3, 0, 0, 1]], [[0, 1, 0, 2, 3, 0, 1, 2]]]
+    _, mbs = opl.preprocess_data_list(vl_samples(), False, packing=True, max_token_in_seq=9, model_type="vlm")
+    assert len(mbs) == 1 and mbs[0]["position_ids"].tolist() == want_packed
+    assert mbs[0]["all_tokens"].tolist() == [[1, 2, 3, 4, 5, 6, 1, 2]] and mbs[0]["labels"].tolist() == [[2, 3, 4, 5, 6, 1, 2, 1]]
+    _, mbs = opl.preprocess_data_list(vl_samples(), False, packing=True, max_token_in_seq=9, model_type="vlm",
+                                      prepend_text_position_channel=True)
+    assert mbs[0]["position_ids"].tolist() == [want_packed[0]] + want_packed
+    # the model is called with the image tensors (policy_trainer.py:206-214)
+    seen = {}
+
+    def model(ids, pos, pixel_values=None, image_grid_thw=None):
+        seen.update(pos=tuple(pos.shape), pix=tuple(pixel_values.shape), grid=image_grid_thw.tolist())
+        return ToyModel()(ids, pos)
+    opl.forward_step(model, vl_samples(), packing=True, trainable=True, max_token_in_seq=9, model_type="vlm")
+    assert seen == {"pos": (3, 1, 8), "pix": (6, 3), "grid": [[1, 2, 2], [1, 2, 1]]}
