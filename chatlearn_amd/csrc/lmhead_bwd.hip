@@ -715,6 +715,12 @@ static int launch_gemm_one(const void* A, int64_t a_kslabs, int M, const void* B
   if (g.k_split == 1 && n_fixed <= cus && g.n_mt * g.n_nt >= 4 * cus && K >= 2 * slab) {
     g.n_walk = cus / n_fixed;
     if (g.n_walk > n_moving) g.n_walk = n_moving;
+    // A walk is as long as its longest run; one workgroup per tile takes ceil(tiles / CUs) rounds.  Streaming the K
+    // loops into each other is worth a few per cent, not a whole extra tile period (H = 7168: 28 x 64 tiles are 7
+    // rounds exactly, while 9 walks over 64 tiles make runs of 7 and 8).
+    const long walk_periods = (n_moving + g.n_walk - 1) / g.n_walk;
+    const long plain_rounds = ((long)g.n_mt * g.n_nt + cus - 1) / cus;
+    if (walk_periods * 100 > plain_rounds * 104) g.n_walk = 0;
   }
   int grid = ((g.n_walk > 0 ? g.n_walk * n_fixed : g.n_mt * g.n_nt * g.k_split) + 7) / 8 * 8;
   hipLaunchKernelGGL((gemm_nt_kernel<T, OutT, kMContig>), dim3(grid), dim3(Tile::kThreads), Tile::kLdsBytes, stream, g);
