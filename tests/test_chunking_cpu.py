@@ -123,3 +123,30 @@ def test_library_launch_plans():
     assert ops.dhidden_launch_plan(12126, 4096, V, torch.bfloat16) == (0, 1)
     assert ops.dhidden_launch_plan(12700, 4096, V, torch.bfloat16) == (48, 8)
     assert ops.dhidden_launch_plan(1458, 1024, V, torch.float32) == (0, 10)                # 24 tiles: 10 K ranges fill 240 CUs
+
+
+def test_chunk_choice_on_random_layouts_is_always_a_partition():
+    """head_step_chunks with the launch-cost choice switched on: whatever it picks is a partition into ranges
+    within the bound (or single longer sequences), ending on sequence boundaries when asked to."""
+    from chatlearn_amd.fused import head_step_chunks
+    rng = random.Random(5)
+    for _ in range(300):
+        T = rng.randint(1, 40000)
+        cap = rng.choice([256, 1000, 4096, 8192, 17408])
+        seq = rng.random() < 0.5
+        cu = sorted({0, T} | {rng.randint(1, T) for _ in range(rng.randint(0, 12))})
+        mask = None
+        if rng.random() < 0.6:
+            mask = (torch.rand(T, generator=torch.Generator().manual_seed(rng.randint(0, 1 << 30))) < rng.choice([0.1, 0.7, 1.0])).int()
+        ranges = head_step_chunks(T, cap, seq, cu, mask, shape=(rng.choice([1024, 2048, 4096, 7168]), rng.choice([32000, 129280, 151936])))
+        assert ranges[0][0] == 0 and ranges[-1][1] == T
+        assert all(a[1] == b[0] for a, b in zip(ranges, ranges[1:])) and all(hi > lo for lo, hi in ranges)
+        cum = None if mask is None else np.concatenate([[0], np.cumsum(mask.numpy() != 0)])
+        for lo, hi in ranges:
+            rows = (hi - lo) if cum is None else int(cum[hi] - cum[lo])
+            if seq and len(ranges) > 1:
+                assert hi in cu
+                if rows > cap:
+                    assert not any(lo < x < hi and (cum is None or cum[lo] < cum[x] < cum[hi]) for x in cu)
+            elif not seq:
+                assert rows <= cap
