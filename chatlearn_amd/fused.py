@@ -129,7 +129,7 @@ class _FusedHead(torch.autograd.Function):
         zbuf = row_map = None
         live = None            # device int64 positions of the live rows; None: every row
         n_live = T
-        if keep_rows is not None and T > 0:
+        if T > 0:
             if mask_host is not None:
                 live_h = _host_live_rows(mask_host, T)          # no device value is read back
                 n_live = int(live_h.size)
@@ -239,11 +239,13 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     h2 = hidden.reshape(-1, hidden.shape[-1])
     needs_grad = torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad)
     keep = _resolve_keep(keep_logits_rows, weight.shape[0], hidden.dtype) if needs_grad else None
-    mask = None
-    if keep is not None and loss_mask is not None and loss_mask_host is None:
-        mask = loss_mask.reshape(-1).to(torch.int32)
+    mask = host = None
+    if needs_grad:                 # the masks only matter to the backward (and to which rows keep their logits)
+        host = loss_mask_host
+        if loss_mask is not None and host is None:
+            mask = loss_mask.reshape(-1).to(torch.int32)
     lp, ent = _FusedHead.apply(h2, weight, labels.reshape(-1), float(temperature), bool(need_entropy), dweight_buffer,
-                               keep, mask, loss_mask_host if keep is not None else None)
+                               keep, mask, host)
     lp = lp.reshape(lead)
     ent = ent.reshape(lead) if need_entropy else None
     return lp, ent

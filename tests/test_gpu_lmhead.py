@@ -169,7 +169,8 @@ def test_autograd_kept_logits_mask_hint_and_second_backward(dev, dtype):
              ("100 of 300 rows kept, no mask", dict(keep_logits_rows=100)),
              ("64 unmasked rows kept, the others recomputed", dict(keep_logits_rows=64, loss_mask=mask.to(dev))),
              ("64 kept, host mask", dict(keep_logits_rows=64, loss_mask_host=mask)),
-             ("256 kept (one block), no mask", dict(keep_logits_rows=256)))
+             ("256 kept (one block), no mask", dict(keep_logits_rows=256)),
+             ("nothing kept, host mask: only the unmasked rows are recomputed", dict(keep_logits_rows=None, loss_mask_host=mask)))
     assert int(mask.sum()) > 64
     for name, kw in cases:
         gh, gw = grads(**kw)
