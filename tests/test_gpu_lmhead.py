@@ -386,3 +386,46 @@ def test_kept_logits_beyond_the_half_range_stay_finite(dev):
     assert_close_rel(dh[others], dh0[others], 2 ** -6, "dhidden of the other tokens, kept against recomputed")
     # token 3's hidden row is zero outside column 0, so it reaches dW through that column only
     assert_close_rel(dw[:, 1:], dw0[:, 1:], 2 ** -6, "dweight outside the saturated token's column")
+
+
+def _random_shapes(n, seed):
+    """Seeded shapes that end anywhere inside a tile: tokens 1..1400, vocabulary 2..3300, H a multiple of the slab."""
+    import random
+    rnd = random.Random(seed)
+    out = []
+    for i in range(n):
+        dtype = torch.bfloat16 if i % 3 else torch.float32
+        slab = 64 if dtype == torch.bfloat16 else 32
+        out.append((rnd.randint(1, 1400), slab * rnd.randint(1, 6), rnd.randint(2, 3300), dtype,
+                    rnd.choice([1.0, 0.6, 1.7]), rnd.choice([None, 256, 512]), rnd.random() < 0.5))
+    return out
+
+
+@pytest.mark.parametrize("T,H,V,dtype,temp,chunk,with_entropy", _random_shapes(14, seed=2024))
+def test_random_shapes_both_backward_routes(dev, T, H, V, dtype, temp, chunk, with_entropy):
+    """Random shapes, temperatures, chunkings and gradient masks: forward and both backward routes against the
+    oracle's float64 closed form, to the tolerance of the dtype."""
+    from chatlearn_amd import ops
+    hidden, weight, labels = _inputs(T, H, V, dtype, seed=T * 31 + V, w_std=0.15)
+    g = torch.Generator().manual_seed(T + H + V)
+    g_lp = torch.randn(T, generator=g)
+    g_lp[torch.rand(T, generator=g) < 0.4] = 0.0
+    g_ent = torch.randn(T, generator=g) * 0.1 if with_entropy else None
+    if with_entropy:
+        g_ent[g_lp == 0] = 0.0          # a masked token carries neither gradient
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    r = RTOL[dtype]
+    rlp, rent, _, rlse = osm.fused_head_forward(hidden, weight, labels, temp, torch.float64)
+    rdh, rdw = osm.fused_head_backward_closed_form(hidden, weight, labels, g_lp, g_ent, temp)
+    zbuf = ops.saved_logits_buffer(T, V, dtype, dev)
+    for saved in (None, zbuf):
+        lp, ent, _, lse = ops.lmhead_forward(hd, wd, ld, temp, need_entropy=True, saved_logits=saved)
+        assert_close_rel(lp, rlp, r, "logprob")
+        assert_close_rel(ent, rent, r, "entropy")
+        # the kept-logits route transforms the whole buffer in one go: chunking applies to the recompute route
+        dh, dw = ops.lmhead_backward(hd, wd, ld, lse, ent, g_lp.to(dev), g_ent.to(dev) if with_entropy else None, temp,
+                                     saved_logits=saved, chunk_tokens=chunk if saved is None else None)
+        route = "kept logits" if saved is not None else "recompute"
+        assert_close_rel(dh, rdh, r, f"dhidden ({route})")
+        assert_close_rel(dw, rdw, r, f"dweight ({route})")
+        assert (dh[g_lp.to(dev) == 0] == 0).all(), "rows without a gradient get an exactly zero dhidden"
