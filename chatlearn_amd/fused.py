@@ -23,10 +23,16 @@ from ._lib import LOSS_GRPO, LOSS_GSPO
 
 
 # Memory one chunk's kept logits may take (they are turned into d(logits) in place; the backward's transposed
-# copy takes as much again).  The bound is on bytes, whatever the hidden size: 17408 rows of a 152k
-# vocabulary, 20736 rows of a 129k one, in 16-bit elements.
-DEFAULT_KEEP_LOGITS_BYTES = 5 << 30
+# copy takes as much again).  The bound is on bytes, whatever the hidden size: 35328 rows of a 152k
+# vocabulary, 41472 rows of a 129k one, in 16-bit elements - a 32768-token micro-batch in one chunk.  Only
+# what a micro-batch needs is allocated.
+DEFAULT_KEEP_LOGITS_BYTES = 10 << 30
 AUTO = "auto"
+# Hidden states one chunk of the head step may span: the size of the last-level cache (18724 tokens at
+# H = 7168, 32768 at H = 4096, in 16-bit elements).  The forward re-reads a chunk's hidden states once per
+# vocabulary split; past this size those reads go to HBM (measured at H = 7168: one chunk of 32768 tokens
+# runs its forward 8 % slower than two of 16384).
+CHUNK_HIDDEN_BYTES = 256 << 20
 
 
 def default_keep_rows(V: int, dtype) -> int:
@@ -261,8 +267,10 @@ def _token_chunks(T, chunk_rows, seq_bounds, live_cum=None, n_ranges=None):
     on a multiple of 256 tokens where the bound leaves room for that.  ``n_ranges`` asks for that many
     ranges instead of the fewest (it is raised to the fewest when smaller)."""
     total = T if live_cum is None else int(live_cum[T])
-    if chunk_rows is None or chunk_rows >= total or T == 0:
+    if T == 0 or ((chunk_rows is None or chunk_rows >= total) and (n_ranges is None or n_ranges <= 1)):
         return [(0, T)]
+    if chunk_rows is None or chunk_rows > total:
+        chunk_rows = max(total, 1)                                 # no bound on the rows: only the number of ranges is asked for
     wt = (lambda pos: pos) if live_cum is None else (lambda pos: int(live_cum[pos]))
 
     def first_with(rows):       # smallest position with at least `rows` rows before it
@@ -345,22 +353,30 @@ def _launch_cost(chunks, live_cum, H, V, dtype=torch.bfloat16, cus=256):
 
 
 def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask_host=None, shape=None,
-                     dtype=torch.bfloat16):
+                     dtype=torch.bfloat16, chunk_hidden_bytes=None):
     """The token ranges ``grpo_head_step`` walks: at most ``keep_logits_chunk`` kept rows each.  Only
     unmasked rows keep their logits, so with the mask known on the host (``loss_mask_host``, given when
     masked rows are skipped) the bound counts those; the sequence-level loss needs ranges that end on
     sequence boundaries (``cu_seqlens``: host list or device tensor, read only when a split is needed).
     With ``shape`` = (H, V) the number of ranges is the fewest the bound allows or up to two more,
     whichever fills the CUs best over the forward and the two backward GEMMs (a launch takes whole
-    rounds of one workgroup per CU; ragged sequence-aligned ranges can leave a round nearly empty)."""
+    rounds of one workgroup per CU; ragged sequence-aligned ranges can leave a round nearly empty).
+    ``chunk_hidden_bytes`` (with ``shape``) also bounds the hidden states of a range: the forward re-reads a
+    range's hidden states once per vocabulary tile, and serves those reads from the last-level cache only
+    while they fit there beside the weight that streams through."""
     live_cum = None
     if loss_mask_host is not None and T > 0:
         live_cum = np.concatenate([[0], np.cumsum(loss_mask_host.reshape(-1).numpy() != 0, dtype=np.int64)])
     rows_total = T if live_cum is None else int(live_cum[T])
+    min_ranges = 1
+    if chunk_hidden_bytes and shape is not None and T > 0:
+        row_bytes = shape[0] * (2 if dtype != torch.float32 else 4)
+        min_ranges = max(1, -(-(T * row_bytes) // int(chunk_hidden_bytes)))
+    split = (keep_logits_chunk is not None and keep_logits_chunk < rows_total) or min_ranges > 1
     bounds = None
-    if keep_logits_chunk is not None and keep_logits_chunk < rows_total and sequence_level:
+    if split and sequence_level:
         bounds = cu_seqlens.tolist() if isinstance(cu_seqlens, torch.Tensor) else list(cu_seqlens)
-    fewest = _token_chunks(T, keep_logits_chunk, bounds, live_cum)
+    fewest = _token_chunks(T, keep_logits_chunk, bounds, live_cum, n_ranges=min_ranges if min_ranges > 1 else None)
     if shape is None or len(fewest) == 1:
         return fewest
     H, V = shape
@@ -383,7 +399,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                    keep_logits_chunk=AUTO, cu_seqlens_host=None,
                    skip_masked_rows=True, skip_masked_forward=False, weight_t_cache: Optional[dict] = None,
                    stage_hook=None, loss_mask_host: Optional[torch.Tensor] = None,
-                   workspace_cache: Optional[dict] = None):
+                   workspace_cache: Optional[dict] = None, chunk_hidden_bytes: Optional[int] = CHUNK_HIDDEN_BYTES):
     """Forward + loss + backward of the head for one packed micro-batch, no autograd graph.
 
     Mirrors policy_trainer.py:216-286 on packed rows: returns a dict with the
@@ -414,6 +430,9 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     it the unmasked rows of every chunk are found on the host and sent over asynchronously; without it
     they are found on the device, which costs one host round trip per chunk for their count.
 
+    ``chunk_hidden_bytes``: a chunk's hidden states are also kept below this many bytes (default
+    ``CHUNK_HIDDEN_BYTES``; ``None``: no such bound), because the forward re-reads them once per vocabulary tile.
+
     ``weight_t_cache``: a dict the caller keeps while ``weight`` does not change (the micro-batches
     of one optimizer step).  The first backward leaves the transposed weight in it and later calls
     reuse it instead of transposing again; the caller clears it after updating the weight.
@@ -438,7 +457,8 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
         raise ValueError(f"loss_mask_host must be a CPU copy of loss_mask with {T} entries")
     chunks = head_step_chunks(T, keep_logits_chunk, use_group_sequence_policy,
                               cu_seqlens_host if cu_seqlens_host is not None else cu_seqlens,
-                              loss_mask_host if skip else None, shape=(hidden.shape[1], V), dtype=hidden.dtype)
+                              loss_mask_host if skip else None, shape=(hidden.shape[1], V), dtype=hidden.dtype,
+                              chunk_hidden_bytes=chunk_hidden_bytes if keep_logits_chunk is not None else None)
     zbuf = None
     rows_of = None
     if skip and loss_mask_host is not None and T > 0:

@@ -138,7 +138,8 @@ def test_chunk_choice_on_random_layouts_is_always_a_partition():
         mask = None
         if rng.random() < 0.6:
             mask = (torch.rand(T, generator=torch.Generator().manual_seed(rng.randint(0, 1 << 30))) < rng.choice([0.1, 0.7, 1.0])).int()
-        ranges = head_step_chunks(T, cap, seq, cu, mask, shape=(rng.choice([1024, 2048, 4096, 7168]), rng.choice([32000, 129280, 151936])))
+        ranges = head_step_chunks(T, cap, seq, cu, mask, shape=(rng.choice([1024, 2048, 4096, 7168]), rng.choice([32000, 129280, 151936])),
+                                  chunk_hidden_bytes=rng.choice([None, 64 << 20, 256 << 20]))
         assert ranges[0][0] == 0 and ranges[-1][1] == T
         assert all(a[1] == b[0] for a, b in zip(ranges, ranges[1:])) and all(hi > lo for lo, hi in ranges)
         cum = None if mask is None else np.concatenate([[0], np.cumsum(mask.numpy() != 0)])
@@ -150,3 +151,27 @@ def test_chunk_choice_on_random_layouts_is_always_a_partition():
                     assert not any(lo < x < hi and (cum is None or cum[lo] < cum[x] < cum[hi]) for x in cu)
             elif not seq:
                 assert rows <= cap
+
+
+def test_bound_on_a_chunk_s_hidden_states():
+    """Besides the bound on the kept rows, a chunk's hidden states stay below ``chunk_hidden_bytes``: 32768 tokens
+    at H = 7168 (448 MiB in 16-bit elements) are cut in two although every row's logits would fit one chunk,
+    at H = 2048 (128 MiB) they are one chunk; fp32 counts 4 bytes per element; sequence-level ranges still end
+    on sequence boundaries; without a shape or a bound nothing is cut."""
+    from chatlearn_amd.fused import CHUNK_HIDDEN_BYTES, default_keep_rows, head_step_chunks
+    assert CHUNK_HIDDEN_BYTES == 256 << 20
+    keep = default_keep_rows(129280, torch.bfloat16)
+    assert keep >= 32768
+    assert head_step_chunks(32768, keep, False, None, None, shape=(7168, 129280), chunk_hidden_bytes=CHUNK_HIDDEN_BYTES) == \
+        [(0, 16384), (16384, 32768)]
+    assert head_step_chunks(32768, keep, False, None, None, shape=(7168, 129280)) == [(0, 32768)]
+    assert head_step_chunks(32768, keep, False, None, None, shape=None, chunk_hidden_bytes=CHUNK_HIDDEN_BYTES) == [(0, 32768)]
+    assert head_step_chunks(32768, default_keep_rows(151936, torch.bfloat16), False, None, None, shape=(2048, 151936),
+                            chunk_hidden_bytes=CHUNK_HIDDEN_BYTES) == [(0, 32768)]
+    assert len(head_step_chunks(32768, 1 << 20, False, None, None, shape=(4096, 32000), dtype=torch.float32,
+                                chunk_hidden_bytes=CHUNK_HIDDEN_BYTES)) == 2
+    cu = [0, 5000, 9000, 15000, 21000, 26000, 30000, 32768]
+    mask = (torch.arange(32768) % 4 != 0).int()
+    ranges = head_step_chunks(32768, keep, True, cu, mask, shape=(7168, 129280), chunk_hidden_bytes=CHUNK_HIDDEN_BYTES)
+    assert len(ranges) >= 2 and ranges[0][0] == 0 and ranges[-1][1] == 32768 and all(hi in cu for _, hi in ranges)
+    assert all(a[1] == b[0] for a, b in zip(ranges, ranges[1:]))
