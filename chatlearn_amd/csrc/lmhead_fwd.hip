@@ -34,6 +34,7 @@ struct FwdParams {
   const int32_t* z_row_map;  // optional [T]: destination row per token, < 0: not stored
   int z_rows;                // rows of z_out; mapped rows outside [0, z_rows) are not stored
   float4* part;  // [n_split][T]: (max raw, sum 2^{(z-max) c}, sum 2^{(z-max) c} z raw, target raw)
+  int xcd_wgs;   // > 0: launch of several rounds, see xcd_round_remap
 };
 
 // 16 bytes of kept logits from consecutive accumulator registers.
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(kHeadThreads) void lmhead_fwd_kernel(FwdParams p) {
   constexpr int MI = Tile::MI, NI = Tile::NI, WM = Tile::WM, WN = Tile::WN;
   extern __shared__ __align__(16) char lds[];
 
-  const int item = xcd_remap(blockIdx.x, gridDim.x);
+  const int item = work_item(p.xcd_wgs);
   if (item >= p.n_tb * p.n_split) return;
   int vs, tb;
   grouped_tile(item, p.n_split, p.n_tb, 4, vs, tb);
@@ -345,9 +346,9 @@ static int launch_fwd(const clgrpo_lmhead_fwd_args* a, hipStream_t stream, int64
   constexpr int lds_bytes = Tile::kLdsBytes;
   int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(&lmhead_fwd_kernel<T, STORE_Z>), lds_bytes, "lmhead_fwd_kernel");
   if (rc) return rc;
-  int grid = p.n_tb * p.n_split;
-  grid = (grid + 7) / 8 * 8;
-  hipLaunchKernelGGL((lmhead_fwd_kernel<T, STORE_Z>), dim3(grid), dim3(Tile::kThreads), lds_bytes, stream, p);
+  const ItemGrid ig = item_grid(p.n_tb * p.n_split, device_cu_count());
+  p.xcd_wgs = ig.xcd_wgs;
+  hipLaunchKernelGGL((lmhead_fwd_kernel<T, STORE_Z>), dim3(ig.grid), dim3(Tile::kThreads), lds_bytes, stream, p);
   rc = check_launch("lmhead_fwd_kernel");
   if (rc) return rc;
   FinalizeParams f;

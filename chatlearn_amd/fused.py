@@ -28,11 +28,10 @@ from ._lib import LOSS_GRPO, LOSS_GSPO
 # what a micro-batch needs is allocated.
 DEFAULT_KEEP_LOGITS_BYTES = 10 << 30
 AUTO = "auto"
-# Hidden states one chunk of the head step may span: the size of the last-level cache (18724 tokens at
-# H = 7168, 32768 at H = 4096, in 16-bit elements).  The forward re-reads a chunk's hidden states once per
-# vocabulary split; past this size those reads go to HBM (measured at H = 7168: one chunk of 32768 tokens
-# runs its forward 8 % slower than two of 16384).
-CHUNK_HIDDEN_BYTES = 256 << 20
+# Optional second bound, on the hidden states one chunk of the head step spans (None: off).  It paid at
+# H = 7168 (one chunk of 32768 tokens against two of 16384) only while the forward's workgroups of different
+# XCDs worked on vocabulary ranges far apart; with the forward's present mapping one chunk is as fast.
+CHUNK_HIDDEN_BYTES = None
 
 
 def default_keep_rows(V: int, dtype) -> int:
@@ -361,9 +360,7 @@ def head_step_chunks(T, keep_logits_chunk, sequence_level, cu_seqlens, loss_mask
     With ``shape`` = (H, V) the number of ranges is the fewest the bound allows or up to two more,
     whichever fills the CUs best over the forward and the two backward GEMMs (a launch takes whole
     rounds of one workgroup per CU; ragged sequence-aligned ranges can leave a round nearly empty).
-    ``chunk_hidden_bytes`` (with ``shape``) also bounds the hidden states of a range: the forward re-reads a
-    range's hidden states once per vocabulary tile, and serves those reads from the last-level cache only
-    while they fit there beside the weight that streams through."""
+    ``chunk_hidden_bytes`` (with ``shape``) also bounds the hidden states of a range."""
     live_cum = None
     if loss_mask_host is not None and T > 0:
         live_cum = np.concatenate([[0], np.cumsum(loss_mask_host.reshape(-1).numpy() != 0, dtype=np.int64)])
@@ -430,8 +427,8 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     it the unmasked rows of every chunk are found on the host and sent over asynchronously; without it
     they are found on the device, which costs one host round trip per chunk for their count.
 
-    ``chunk_hidden_bytes``: a chunk's hidden states are also kept below this many bytes (default
-    ``CHUNK_HIDDEN_BYTES``; ``None``: no such bound), because the forward re-reads them once per vocabulary tile.
+    ``chunk_hidden_bytes``: a chunk's hidden states are also kept below this many bytes (``None``, the
+    default: no such bound).
 
     ``weight_t_cache``: a dict the caller keeps while ``weight`` does not change (the micro-batches
     of one optimizer step).  The first backward leaves the transposed weight in it and later calls

@@ -154,12 +154,12 @@ def test_chunk_choice_on_random_layouts_is_always_a_partition():
 
 
 def test_bound_on_a_chunk_s_hidden_states():
-    """Besides the bound on the kept rows, a chunk's hidden states stay below ``chunk_hidden_bytes``: 32768 tokens
+    """Besides the bound on the kept rows, a chunk's hidden states stay below ``chunk_hidden_bytes`` when one is given: 32768 tokens
     at H = 7168 (448 MiB in 16-bit elements) are cut in two although every row's logits would fit one chunk,
     at H = 2048 (128 MiB) they are one chunk; fp32 counts 4 bytes per element; sequence-level ranges still end
     on sequence boundaries; without a shape or a bound nothing is cut."""
-    from chatlearn_amd.fused import CHUNK_HIDDEN_BYTES, default_keep_rows, head_step_chunks
-    assert CHUNK_HIDDEN_BYTES == 256 << 20
+    from chatlearn_amd.fused import default_keep_rows, head_step_chunks
+    CHUNK_HIDDEN_BYTES = 256 << 20
     keep = default_keep_rows(129280, torch.bfloat16)
     assert keep >= 32768
     assert head_step_chunks(32768, keep, False, None, None, shape=(7168, 129280), chunk_hidden_bytes=CHUNK_HIDDEN_BYTES) == \
