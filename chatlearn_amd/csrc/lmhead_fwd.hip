@@ -301,26 +301,36 @@ __global__ void lmhead_fwd_finalize_kernel(FinalizeParams p) {
 
 // Split of the vocabulary tiles over workgroups.  A workgroup walks ceil(n_vt / n_split) tiles for
 // one block of 256 tokens; with each CU holding one workgroup a launch takes
-// ceil(n_tb * n_split / CUs) rounds, so its cost in tile periods is rounds * tiles-per-workgroup.  At
-// least four splits when possible: the workgroups of an XCD then form a 4-row block sharing operands.
-// The launch over n_tb token blocks: returns its cost in sixteenths of a tile period (small penalties break
-// ties).  Many splits and several rounds are fine (65 token blocks: 35 splits of 17 tiles, 9 rounds = 153 tile
+// ceil(n_tb * n_split / CUs) rounds, so its cost in tile periods is rounds * tiles-per-workgroup.
+// Many splits and several rounds are fine (65 token blocks: 35 splits of 17 tiles, 9 rounds = 153 tile
 // periods against the ideal 151), so the plan stays within a few per cent of n_tb * n_vt / CUs tile periods
-// from about 7 token blocks on.  `cus` <= 0 plans for a 256-CU device.
+// from about 7 token blocks on.  Two smaller terms, both measured on launches of equal tile periods:
+//  - the splits are handed out in groups of 4 (the workgroups of an XCD then form a block of 4 splits x
+//    CUs/32 token blocks that shares operand slabs in the XCD's L2: 4 + 8 = 12 slabs per step for 32 tiles).
+//    A last group of w < 4 splits makes blocks of w x 32/w, w + 32/w slabs per step; the time grows by about
+//    0.11 of that excess (65536 tokens at H = 4096: 5 splits 63.4 ms, 2 splits 64.2 ms, 6 splits 61.3 ms
+//    against 60.6 ms with 4 or 60.9 ms with 8);
+//  - every run of tiles starts with a K loop whose first slabs nothing has requested in advance and ends
+//    with its partial record: 0.3 tile periods (32768 tokens at H = 7168: 22 splits x 23 tiles 45.2 ms, 4
+//    x 127 or 8 x 64 tiles 44.3 - 44.6 ms).
+// Returns the launch's cost in sixteenths of a tile period.  `cus` <= 0 plans for a 256-CU device.
 static long fwd_single_cost(int n_tb, int n_vt, int cus, int& n_split, int& tiles_per_split) {
   if (cus <= 0) cus = 256;
+  const double xcd_wgs = cus / 8.0, full_block = 4.0 + xcd_wgs / 4.0;
   int best = 1;
-  long best_cost = -1;
+  double best_cost = -1.0;
   for (int sp = 1; sp <= kMaxFwdSplits && sp <= n_vt; ++sp) {
     const int tps = (n_vt + sp - 1) / sp;
     const int eff_sp = (n_vt + tps - 1) / tps;
     const long rounds = ((long)n_tb * eff_sp + cus - 1) / cus;
-    long cost = rounds * tps * 16 + (sp < 4 ? 8 : 0) + eff_sp / 8;
+    const int rem = eff_sp % 4;
+    const double excess = rem ? (double)rem / eff_sp * ((rem + xcd_wgs / rem) / full_block - 1.0) : 0.0;
+    const double cost = (double)rounds * (tps + 0.3) * 16.0 * (1.0 + 0.11 * excess) + eff_sp * 0.01;
     if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = sp; }
   }
   tiles_per_split = (n_vt + best - 1) / best;
   n_split = (n_vt + tiles_per_split - 1) / tiles_per_split;
-  return best_cost;
+  return (long)(best_cost + 0.5);
 }
 
 template <typename T, bool STORE_Z>
