@@ -604,7 +604,8 @@ def other_config(name, device, steps, warmup):
                             f"{'bf16' if cfg.dtype == torch.bfloat16 else 'fp32'}"
                             f"{' temperature ' + str(cfg.temperature) if cfg.temperature != 1.0 else ''}",
                 "forward_kernel_frac_of_peak": round(fwd_tf / peak_of(cfg), 4),
-                "forward_launches": len(rec["token_chunks"])})
+                "forward_launches": len(rec["token_chunks"]),
+                "forward_traffic_bytes_per_launch": measured_traffic(cfg.name, max(rec["token_chunks"]), keep)})
     rec["tokens_per_s"] = round(rec["tokens_per_s"], 1)
     rec["ms_per_step"] = round(rec["ms_per_step"], 3)
     rec["step_mfma_frac_executed"] = round(rec["step_mfma_frac_executed"], 4)
