@@ -29,7 +29,7 @@ sys.path.insert(0, ROOT)
 
 from chatlearn_amd import _lib, ops, synthetic  # noqa: E402
 from chatlearn_amd._lib import LOSS_GRPO, LOSS_GSPO  # noqa: E402
-from chatlearn_amd.fused import CHUNK_HIDDEN_BYTES, default_keep_rows, grpo_head_step, head_step_chunks  # noqa: E402
+from chatlearn_amd.fused import default_keep_rows, grpo_head_step, head_step_chunks  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3
@@ -326,8 +326,7 @@ def gemm_kernels(w, keep, reps=3):
     whole backward of the chunk and the backward without that output (what remains in either is the
     d(logits) pass and a transpose)."""
     cfg = w.cfg
-    chunks = head_step_chunks(w.T, keep, cfg.loss == "gspo", w.cu_host, w.mask_host, shape=(cfg.H, cfg.V), dtype=cfg.dtype,
-                              chunk_hidden_bytes=CHUNK_HIDDEN_BYTES if keep is not None else None)
+    chunks = head_step_chunks(w.T, keep, cfg.loss == "gspo", w.cu_host, w.mask_host, shape=(cfg.H, cfg.V), dtype=cfg.dtype)
     lo, hi = max(chunks, key=lambda c: c[1] - c[0])
     n = hi - lo
     dev = w.device

@@ -28,10 +28,6 @@ from ._lib import LOSS_GRPO, LOSS_GSPO
 # what a micro-batch needs is allocated.
 DEFAULT_KEEP_LOGITS_BYTES = 10 << 30
 AUTO = "auto"
-# Optional second bound, on the hidden states one chunk of the head step spans (None: off).  It paid at
-# H = 7168 (one chunk of 32768 tokens against two of 16384) only while the forward's workgroups of different
-# XCDs worked on vocabulary ranges far apart; with the forward's present mapping one chunk is as fast.
-CHUNK_HIDDEN_BYTES = None
 
 
 def default_keep_rows(V: int, dtype) -> int:
@@ -396,7 +392,7 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
                    keep_logits_chunk=AUTO, cu_seqlens_host=None,
                    skip_masked_rows=True, skip_masked_forward=False, weight_t_cache: Optional[dict] = None,
                    stage_hook=None, loss_mask_host: Optional[torch.Tensor] = None,
-                   workspace_cache: Optional[dict] = None, chunk_hidden_bytes: Optional[int] = CHUNK_HIDDEN_BYTES):
+                   workspace_cache: Optional[dict] = None, chunk_hidden_bytes: Optional[int] = None):
     """Forward + loss + backward of the head for one packed micro-batch, no autograd graph.
 
     Mirrors policy_trainer.py:216-286 on packed rows: returns a dict with the
@@ -428,7 +424,8 @@ def grpo_head_step(hidden, weight, labels, old_logprob, ref_logprob, advantages,
     they are found on the device, which costs one host round trip per chunk for their count.
 
     ``chunk_hidden_bytes``: a chunk's hidden states are also kept below this many bytes (``None``, the
-    default: no such bound).
+    default: no such bound).  It paid at H = 7168 (two chunks of 16384 tokens against one of 32768) only while
+    the forward's workgroups of different XCDs worked on vocabulary ranges far apart.
 
     ``weight_t_cache``: a dict the caller keeps while ``weight`` does not change (the micro-batches
     of one optimizer step).  The first backward leaves the transposed weight in it and later calls
