@@ -140,6 +140,23 @@ def test_other_benchmark_configs_at_full_size(dev, name):
         assert col.abs().max() < 5e-3 * out["dweight"].abs().sum(0).max()   # sum_v dz = 0
         assert out["rows_projected_bwd"] == int(mask.sum())
         assert math.isfinite(float(out["total_loss"]))
+        # the default bound keeps the whole micro-batch in one chunk; a bound of 12288 rows cuts it into three or
+        # more (on sequence boundaries for the sequence-level loss): same loss, same gradients
+        assert len(out["token_chunks"]) == 1
+        dh1, dw1, loss1 = out["dhidden"].clone(), out["dweight"].clone(), float(out["total_loss"])
+        del out
+        cut = grpo_head_step(hidden, weight, labels, old, old, adv, cu, mask, n_tokens_total=float(mask.sum()),
+                             use_group_sequence_policy=(cfg.loss == "gspo"), pos_clip_ratio=cfg.pos_clip_ratio,
+                             neg_clip_ratio=cfg.neg_clip_ratio, kl_coef=cfg.kl_coef, entropy_coef=cfg.entropy_coef,
+                             temperature=cfg.temperature, cu_seqlens_host=cu.tolist(), keep_logits_chunk=12288)
+        assert len(cut["token_chunks"]) >= 3
+        if cfg.loss == "gspo":
+            ends = set(cu.tolist())
+            assert all(hi in ends for _, hi in cut["token_chunks"])
+        assert float(cut["total_loss"]) == pytest.approx(loss1, rel=1e-5)
+        assert_close_rel(cut["dhidden"], dh1, 1e-2, "dhidden, three chunks against one")
+        assert_close_rel(cut["dweight"], dw1, 1e-2, "dW, three chunks against one")
+        del cut, dh1, dw1
     assert (lp <= 0).all() and (ent > 0).all() and (ent <= math.log(cfg.V) + 1e-3).all()
     assert_close_rel(lp[rows], want[0], 1e-2, "logprob sample")
     assert_close_rel(ent[rows], want[1], 1e-2, "entropy sample")
