@@ -109,6 +109,7 @@ SIGNATURES = {
     "clgrpo_lmhead_fwd": (C.c_int, [C.POINTER(LmheadFwdArgs), vp]),
     "clgrpo_lmhead_fwd_launch_plan": (C.c_int, [i64, i64, i32, vp]),
     "clgrpo_lmhead_bwd_dhidden_plan": (C.c_int, [i64, i64, i64, i32, i32, vp]),
+    "clgrpo_lmhead_bwd_dweight_plan": (C.c_int, [i64, i64, i64, i32, i32, vp]),
     "clgrpo_saved_logits_ld": (i64, [i64]),
     "clgrpo_lmhead_bwd_workspace_bytes": (sz, [i64, i64, i64, i32, i64, i32]),
     "clgrpo_lmhead_bwd": (C.c_int, [C.POINTER(LmheadBwdArgs), vp]),

@@ -63,5 +63,5 @@ int device_cu_count() {
 
 }  // namespace clgrpo
 
-extern "C" int clgrpo_version(void) { return 201; }
+extern "C" int clgrpo_version(void) { return 202; }
 extern "C" const char* clgrpo_last_error_string(void) { return clgrpo::error_buffer(); }

@@ -642,6 +642,61 @@ static size_t dhidden_partial_bytes(int64_t rows, int64_t H, int64_t ldv, int sl
   return plan_dhidden(rows, H, ldv, slab, 256, (size_t)1 << 30).partial_bytes;
 }
 
+// How the dW GEMM (C[m][n], M = vocabulary rows, N = H, K = the chunk's tokens) is launched.  With many more tiles
+// than CUs its workgroups keep one tile of hidden^T and walk runs of vocabulary tiles (see gemm_nt_kernel); the walks
+// are as long as the longest run, so when the vocabulary tiles do not divide by the number of walks the last
+// `n_mt % n_walk` of them keep a sixteenth of the chip busy for a whole tile period (594 tiles on 16 walks: runs of
+// 37 and 38).  The repair is the one of the dhidden GEMM: a bulk launch whose walks are all equally long, and a second
+// launch over the remaining vocabulary tiles cut into K ranges that fill the CUs (fp32 partial tiles, summed by a small
+// pass).  The partials' traffic (written and read once) is priced in, in slab periods of one tile.
+struct DwPlan {
+  int n_walk;        // walks of the (bulk) launch; 0: one workgroup per tile, no bulk / tail split
+  int bulk_mt;       // vocabulary tiles of the bulk launch; 0: one launch over all of them
+  int k_split;       // K ranges of the tail launch
+  size_t partial_bytes;
+};
+
+static DwPlan plan_dweight(int64_t V, int64_t H, int64_t K, int slab, int cus, size_t partial_cap) {
+  DwPlan pl{0, 0, 1, 0};
+  const int n_mt = (int)((V + 255) / 256), n_nt = (int)((H + 255) / 256);
+  if (!(n_nt <= cus && (long)n_mt * n_nt >= 4L * cus && K >= 2 * slab)) return pl;
+  int n_walk = cus / n_nt;
+  if (n_walk > n_mt) n_walk = n_mt;
+  const long walk_periods = (n_mt + n_walk - 1) / n_walk;
+  const long plain_rounds = ((long)n_mt * n_nt + cus - 1) / cus;
+  if (walk_periods * 100 > plain_rounds * 104) return pl;     // one workgroup per tile is the better launch
+  pl.n_walk = n_walk;
+  const int base = n_mt / n_walk, rem = n_mt % n_walk;
+  if (rem == 0 || base == 0) return pl;
+  const long k_slabs = (K + slab - 1) / slab;
+  const int64_t tail_rows = V - (int64_t)(n_mt - rem) * 256;
+  const long tail_tiles = (long)rem * n_nt;
+  // one slab period of a tile is about 1.65 us; the partials move at about 4 TB/s: 6.6 MB per slab period
+  int best_s = 0;
+  double best = 0.0;
+  for (int s = 1; s <= kMaxKSplit; ++s) {
+    const size_t bytes = s > 1 ? (size_t)s * tail_rows * H * sizeof(float) : 0;
+    if (s > 1) {
+      if (bytes > partial_cap || K / s < 8 * slab) break;
+      const int64_t per = round_up64((K + s - 1) / s, slab);
+      if ((int64_t)(s - 1) * per >= K) continue;
+    }
+    const long rounds = (tail_tiles * s + cus - 1) / cus;
+    const double c = (double)rounds * (double)((k_slabs + s - 1) / s) + 2.0 * (double)bytes / 6.6e6 + (s > 1 ? 0.02 : 0.01) * (double)k_slabs;
+    if (best_s == 0 || c < best) { best = c; best_s = s; }
+  }
+  const double now = (double)(base + 1) * (double)k_slabs, two = (double)base * (double)k_slabs + best;
+  if (best_s == 0 || two >= 0.99 * now) return pl;
+  pl.bulk_mt = n_mt - rem;
+  pl.k_split = best_s;
+  pl.partial_bytes = best_s > 1 ? (size_t)best_s * tail_rows * H * sizeof(float) : 0;
+  return pl;
+}
+
+static size_t dweight_partial_bytes(int64_t rows, int64_t H, int64_t V, int slab) {
+  return rows > 0 ? plan_dweight(V, H, round_up64(rows, 64), slab, 256, (size_t)1 << 30).partial_bytes : 0;
+}
+
 struct BwdPlan {
   int64_t ldv;        // K extent of dz / WT (V rounded up to 64)
   int64_t chunk;      // tokens per chunk (multiple of 256 unless >= T)
@@ -664,11 +719,14 @@ static BwdPlan bwd_plan(int64_t T, int64_t H, int64_t V, size_t es, int64_t chun
   pl.off_hidt = off; off += align_up(Hb * pl.ldt * es, 256);
   pl.off_dz = off;   off += saved ? 0 : align_up(Cb * pl.ldv * es, 256);
   pl.off_dzt = off;  off += align_up(Vb * pl.ldt * es, 256);
-  // split-K partials of dhidden: what a full chunk and the shorter last chunk want
+  // split-K partials of the dhidden GEMM and of the dW GEMM's tail (used one after the other): what a full chunk and
+  // the shorter last chunk want
   const int slab = (int)(kRowBytes / es);
-  const size_t part_full = dhidden_partial_bytes(chunk, H, pl.ldv, slab);
-  const size_t part_last = dhidden_partial_bytes(T % chunk, H, pl.ldv, slab);
-  pl.part_bytes = align_up(part_full > part_last ? part_full : part_last, 256);
+  size_t part = 0;
+  for (size_t b : {dhidden_partial_bytes(chunk, H, pl.ldv, slab), dhidden_partial_bytes(T % chunk, H, pl.ldv, slab),
+                   dweight_partial_bytes(chunk, H, V, slab), dweight_partial_bytes(T % chunk, H, V, slab)})
+    if (b > part) part = b;
+  pl.part_bytes = align_up(part, 256);
   pl.off_part = off; off += pl.part_bytes;
   pl.total = off;
   return pl;
@@ -733,13 +791,27 @@ static int launch_gemm_one(const void* A, int64_t a_kslabs, int M, const void* B
   return check_launch("splitk_reduce_kernel");
 }
 
-// C (+)= A B^T; with `partial` (dhidden only) the launch plan of plan_dhidden applies.
+// C (+)= A B^T under the launch plan of its orientation: plan_dhidden (C[n][m], with `partial`) or plan_dweight (C[m][n]).
 template <typename T, typename OutT, bool kMContig>
 static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, int64_t b_kslabs, int N, int K, void* C,
                        int64_t ldc, int accumulate, hipStream_t stream, float* partial = nullptr,
                        size_t partial_bytes = 0) {
   using Tile = HeadTile<T>;
-  if (!(kMContig && partial && partial_bytes))
+  constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;
+  if (!kMContig) {
+    // dW: equally long walks over most vocabulary tiles, the rest cut into K ranges (plan_dweight)
+    const DwPlan dw = plan_dweight(M, N, K, Tile::kSlabK, device_cu_count(), partial ? partial_bytes : 0);
+    if (dw.bulk_mt == 0)
+      return launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, M, B, b_kslabs, N, K, C, ldc, accumulate, stream, nullptr, 0, 1);
+    const int bulk_rows = dw.bulk_mt * 256;
+    int rc = launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, bulk_rows, B, b_kslabs, N, K, C, ldc, accumulate, stream, nullptr, 0, 1);
+    if (rc) return rc;
+    const T* a_tail = static_cast<const T*>(A) + (int64_t)dw.bulk_mt * a_kslabs * kSlabElems;
+    OutT* c_tail = static_cast<OutT*>(C) + (int64_t)bulk_rows * ldc;
+    return launch_gemm_one<T, OutT, kMContig>(a_tail, a_kslabs, M - bulk_rows, B, b_kslabs, N, K, c_tail, ldc, accumulate, stream,
+                                              dw.k_split > 1 ? partial : nullptr, dw.k_split > 1 ? partial_bytes : 0, dw.k_split);
+  }
+  if (!(partial && partial_bytes))
     return launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, M, B, b_kslabs, N, K, C, ldc, accumulate, stream, nullptr, 0, 1);
   const DhPlan pl = plan_dhidden(N, M, K, Tile::kSlabK, device_cu_count(), partial_bytes);
   if (pl.bulk_nt == 0)
@@ -749,7 +821,6 @@ static int launch_gemm(const void* A, int64_t a_kslabs, int M, const void* B, in
   int rc = launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, M, B, b_kslabs, bulk_rows, K, C, ldc, accumulate, stream,
                                               nullptr, 0, 1);
   if (rc) return rc;
-  constexpr int64_t kSlabElems = (int64_t)kBlockRows * Tile::kSlabK;
   const T* b_tail = static_cast<const T*>(B) + (int64_t)pl.bulk_nt * b_kslabs * kSlabElems;
   OutT* c_tail = static_cast<OutT*>(C) + (int64_t)bulk_rows * ldc;
   return launch_gemm_one<T, OutT, kMContig>(A, a_kslabs, M, b_tail, b_kslabs, N - bulk_rows, K, c_tail, ldc, accumulate,
@@ -852,7 +923,8 @@ static int run_bwd(const clgrpo_lmhead_bwd_args* a, hipStream_t stream, int64_t 
       rc = launch_transpose<T>(hidden + c0 * H, H, hidt, ldt, (int)tc, (int)H, stream);
       if (rc) return rc;
       rc = launch_gemm<T, float, false>(dzt, ldt / Tile::kSlabK, (int)V, hidt, ldt / Tile::kSlabK, (int)H, (int)ldt, a->dweight, H,
-                                        (a->accumulate_dweight || c0 > 0) ? 1 : 0, stream);
+                                        (a->accumulate_dweight || c0 > 0) ? 1 : 0, stream,
+                                        reinterpret_cast<float*>(ws + pl.off_part), pl.part_bytes);
       if (rc) return rc;
     }
   }
@@ -875,6 +947,16 @@ extern "C" int clgrpo_lmhead_bwd_dhidden_plan(int64_t rows, int64_t H, int64_t V
   const DhPlan pl = plan_dhidden(rows, H, round_up64(V, 64), slab, cus > 0 ? cus : 256, (size_t)1 << 30);
   out[0] = pl.bulk_nt;
   out[1] = pl.k_split;
+  return CLGRPO_OK;
+}
+
+extern "C" int clgrpo_lmhead_bwd_dweight_plan(int64_t rows, int64_t H, int64_t V, int32_t dtype, int32_t cus, int32_t* out) {
+  if (rows <= 0 || H <= 0 || V <= 0 || out == nullptr || (dtype != CLGRPO_BF16 && dtype != CLGRPO_F32)) return CLGRPO_EINVAL;
+  const int slab = (int)(kRowBytes / dtype_bytes(dtype));
+  const DwPlan pl = plan_dweight(V, H, round_up64(rows, 64), slab, cus > 0 ? cus : 256, (size_t)1 << 30);
+  out[0] = pl.n_walk;
+  out[1] = pl.bulk_mt;
+  out[2] = pl.k_split;
   return CLGRPO_OK;
 }
 

@@ -182,6 +182,15 @@ def dhidden_launch_plan(rows: int, H: int, V: int, dtype, cus: int = 0) -> Tuple
     return int(out[0]), int(out[1])
 
 
+def dweight_launch_plan(rows: int, H: int, V: int, dtype, cus: int = 0) -> Tuple[int, int, int]:
+    """(walks or 0, vocabulary tiles of a first launch of equally long walks or 0, K ranges of the launch over the
+    remaining vocabulary tiles) for the dW contraction over a chunk of ``rows`` tokens."""
+    out = (C.c_int32 * 3)()
+    _lib.check(_lib.lib().clgrpo_lmhead_bwd_dweight_plan(int(rows), int(H), int(V), BF16 if dtype == torch.bfloat16 else F32,
+                                                         int(cus), C.cast(out, C.c_void_p)))
+    return int(out[0]), int(out[1]), int(out[2])
+
+
 def lmhead_forward_workspace_bytes(T: int, H: int, V: int, dtype) -> int:
     """Bytes of scratch one ``lmhead_forward`` call of T tokens needs."""
     return int(_lib.lib().clgrpo_lmhead_fwd_workspace_bytes(T, H, V, BF16 if dtype == torch.bfloat16 else F32))

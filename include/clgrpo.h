@@ -41,8 +41,10 @@ typedef enum { CLGRPO_BF16 = 0, CLGRPO_F32 = 1, CLGRPO_F64 = 2, CLGRPO_U8 = 3 /*
  *                 inputs are IEEE half in the forward's own order; clgrpo_lmhead_fwd_workspace_bytes grew to
  *                 min(ceil(V / 256), 64) * T * 16.
  *   2.00 -> 2.01: clgrpo_lmhead_bwd_workspace_bytes sizes the split-K partials by the GEMM's plan (smaller in
- *                 general); clgrpo_lmhead_fwd_launch_plan and clgrpo_lmhead_bwd_dhidden_plan added. */
-#define CLGRPO_VERSION 201
+ *                 general); clgrpo_lmhead_fwd_launch_plan and clgrpo_lmhead_bwd_dhidden_plan added.
+ *   2.01 -> 2.02: clgrpo_lmhead_bwd_workspace_bytes also covers the partials of the dW GEMM's tail launch (a few
+ *                 tens of MB more for some shapes); clgrpo_lmhead_bwd_dweight_plan added. */
+#define CLGRPO_VERSION 202
 int clgrpo_version(void);
 const char* clgrpo_last_error_string(void);
 
@@ -147,6 +149,12 @@ int clgrpo_lmhead_bwd(const clgrpo_lmhead_bwd_args* a, void* stream);
  * all rows), out[1] = K ranges of the (remaining) launch, whose fp32 partial tiles a second pass sums.
  * Host-side arithmetic only; no counterpart in the reference. */
 int clgrpo_lmhead_bwd_dhidden_plan(int64_t rows, int64_t H, int64_t V, int32_t dtype, int32_t cus, int32_t* out);
+/* How the dW contraction over a chunk of `rows` tokens is launched: out[0] = walks (workgroups that keep one
+ * 256-column tile of hidden^T and walk runs of vocabulary tiles; 0: one workgroup per tile), out[1] = vocabulary
+ * tiles of a first launch whose walks are all equally long (0: one launch over all of them), out[2] = K ranges of
+ * the launch over the remaining vocabulary tiles (fp32 partial tiles, summed by a second pass).
+ * Host-side arithmetic only; no counterpart in the reference. */
+int clgrpo_lmhead_bwd_dweight_plan(int64_t rows, int64_t H, int64_t V, int32_t dtype, int32_t cus, int32_t* out);
 
 /* ------------------------------------------------------------------ *
  * One vocabulary shard of the head (tensor-parallel lm_head: each rank keeps rows

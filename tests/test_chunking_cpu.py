@@ -123,6 +123,17 @@ def test_library_launch_plans():
     assert ops.dhidden_launch_plan(12126, 4096, V, torch.bfloat16) == (0, 1)
     assert ops.dhidden_launch_plan(12700, 4096, V, torch.bfloat16) == (48, 8)
     assert ops.dhidden_launch_plan(1458, 1024, V, torch.float32) == (0, 10)                # 24 tiles: 10 K ranges fill 240 CUs
+    # dW, H = 4096: 16 walks over 594 vocabulary tiles would be runs of 37 and 38; 592 tiles are walked in runs of 37
+    # and the last 2 x 16 tiles are cut into 8 K ranges (256 work items).  Few tiles: one workgroup per tile, no walks
+    assert ops.dweight_launch_plan(12126, 4096, V, torch.bfloat16) == (16, 592, 8)
+    assert ops.dweight_launch_plan(5000, 4096, 32000, torch.bfloat16) == (16, 0, 1)        # 125 tiles, runs of 7 and 8: the 13 left-over tile rows would fill most CUs anyway
+    assert ops.dweight_launch_plan(700, 512, 9001, torch.bfloat16) == (0, 0, 1)
+    for rows, H, vocab in [(32767, 2048, V), (16384, 7168, 129280), (1457, 1024, V), (300, 4096, V), (65536, 4096, V)]:
+        n_walk, bulk, ks = ops.dweight_launch_plan(rows, H, vocab, torch.bfloat16)
+        n_mt = -(-vocab // 256)
+        assert 0 <= bulk < n_mt and 1 <= ks <= 16
+        if bulk:
+            assert n_walk > 0 and bulk % n_walk == 0 and n_mt - bulk < n_walk              # equal runs, fewer tiles left than walks
 
 
 def test_chunk_choice_on_random_layouts_is_always_a_partition():

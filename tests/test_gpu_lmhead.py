@@ -217,11 +217,16 @@ def test_argument_errors(dev):
     assert torch.isfinite(lp[:2]).all() and torch.isnan(lp[2:]).all()
 
 
-def test_backward_weight_gradient_with_walking_workgroups(dev):
+@pytest.mark.parametrize("T", [200, 1100])
+def test_backward_weight_gradient_with_walking_workgroups(dev, T):
     """A weight-gradient GEMM with many more 256 x 256 tiles than CUs runs with workgroups that walk
-    runs of tiles (consecutive K loops streaming into each other); ragged V and T edges included."""
+    runs of tiles (consecutive K loops streaming into each other); ragged V and T edges included.  With 1100
+    tokens the 65 vocabulary tiles are launched as 64 (16 walks of 4) plus one row of tiles cut into K ranges,
+    whose last tile holds 16 valid rows."""
     from chatlearn_amd import ops
-    T, H, V = 200, 4096, 16400
+    H, V = 4096, 16400
+    n_walk, bulk, ks = ops.dweight_launch_plan(T, H, V, torch.bfloat16)
+    assert n_walk == 16 and ((bulk, ks >= 2) == (64, True) if T == 1100 else bulk == 0)
     hidden, weight, labels = _inputs(T, H, V, torch.bfloat16, seed=9, w_std=0.02)
     g = torch.Generator().manual_seed(6)
     g_lp = torch.randn(T, generator=g)
