@@ -323,9 +323,8 @@ def _token_chunks(T, chunk_rows, seq_bounds, live_cum=None, n_ranges=None):
 def _launch_cost(chunks, live_cum, H, V, dtype=torch.bfloat16, cus=256):
     """Relative time of the three GEMM-shaped passes of every chunk, in units of one 256 x 256 tile over one
     K element on one CU: a launch of n work items takes ceil(n / cus) rounds.  Asks the library for its
-    launch plans (vocabulary splits of the forward, bulk / K-split launches of the dhidden GEMM) and mirrors
-    the walking workgroups of the dW GEMM; the passes that do not depend on the cuts (d(logits),
-    transposes) are left out, the read of dW's previous contents by every chunk after the first is counted."""
+    launch plans (vocabulary splits of the forward, bulk / K-split launches of the dhidden and dW GEMMs);
+    the passes that do not depend on the cuts (d(logits), transposes) are left out, the read of dW's previous contents by every chunk after the first is counted."""
     n_vt = -(-V // 256)
     n_ht = -(-H // 256)
     cost = 0.0
@@ -340,8 +339,11 @@ def _launch_cost(chunks, live_cum, H, V, dtype=torch.bfloat16, cus=256):
         if bulk_nt:
             cost += -(-(bulk_nt * n_ht) // cus) * V
         cost += -(-((n_rt - bulk_nt) * n_ht * ks) // cus) * (V / ks)
-        walk = max(1, cus // n_ht)                             # dW: workgroups keep an H tile and walk vocabulary tiles
-        cost += (-(-n_vt // min(walk, n_vt)) if n_vt * n_ht >= 4 * cus else -(-(n_vt * n_ht) // cus)) * rows
+        n_walk, bulk_vt, ks_w = ops.dweight_launch_plan(rows, H, V, dtype, cus)   # dW: walks over vocabulary tiles, K-split tail
+        if bulk_vt:
+            cost += (bulk_vt // n_walk) * rows + -(-((n_vt - bulk_vt) * n_ht * ks_w) // cus) * (rows / ks_w)
+        else:
+            cost += (-(-n_vt // n_walk) if n_walk else -(-(n_vt * n_ht) // cus)) * rows
         if k > 0:
             cost += 0.15 * n_vt * n_ht / cus * 2048            # re-reading dW [V,H] fp32: HBM time in the same unit
     return cost
